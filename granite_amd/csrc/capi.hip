@@ -1,0 +1,440 @@
+// C ABI of libgranite_hip.so: device lifecycle, memory, timing, and the
+// argument checking in front of the kernel launchers.  This and the kernel
+// files are the only code that includes hip_runtime.h; everything above talks
+// to the functions declared in granite_hip.h.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "common.h"
+
+namespace ghip {
+
+Context& ctx() {
+    static Context c;
+    return c;
+}
+
+int ensure_workspace(size_t bytes) {
+    Context& c = ctx();
+    if (bytes <= c.workspace_bytes) return GRANITE_HIP_OK;
+    // Earlier launches may still read the old buffer.
+    GHIP_CHECK(hipStreamSynchronize(c.stream));
+    if (c.workspace) GHIP_CHECK(hipFree(c.workspace));
+    c.workspace = nullptr;
+    c.workspace_bytes = 0;
+    size_t want = bytes + bytes / 4;
+    want = (want + 255) & ~size_t(255);
+    hipError_t e = hipMalloc(&c.workspace, want);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return GRANITE_HIP_ENOMEM;
+    }
+    c.workspace_bytes = want;
+    return GRANITE_HIP_OK;
+}
+
+}  // namespace ghip
+
+using ghip::ctx;
+
+extern "C" {
+
+const char* granite_hip_version(void) { return "granite-hip 0.1 (gfx950)"; }
+
+const char* granite_hip_error_string(int code) {
+    switch (code) {
+        case GRANITE_HIP_OK: return "ok";
+        case GRANITE_HIP_EINVAL: return "InvalidArgument";
+        case GRANITE_HIP_ENOTINIT: return "BackendNotInitialized";
+        case GRANITE_HIP_ENOMEM: return "AllocationFailed";
+        case GRANITE_HIP_EUNSUPPORTED: return "NotImplemented";
+        case GRANITE_HIP_ENULL: return "NullPointer";
+        case GRANITE_HIP_EOVERFLOW: return "InvalidArgument: KV cache overflow";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown error";
+}
+
+int granite_hip_init(int device) {
+    ghip::Context& c = ctx();
+    if (c.initialized) return c.device == device ? GRANITE_HIP_OK : GRANITE_HIP_EINVAL;
+    int count = 0;
+    GHIP_CHECK(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return GRANITE_HIP_EINVAL;
+    GHIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    GHIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        std::fprintf(stderr, "granite_hip: device %d is %s; this library holds gfx950 code only\n",
+                     device, prop.gcnArchName);
+        return GRANITE_HIP_EUNSUPPORTED;
+    }
+    GHIP_CHECK(hipStreamCreateWithFlags(&c.own_stream, hipStreamNonBlocking));
+    c.stream = c.own_stream;
+    c.device = device;
+    c.compute_units = prop.multiProcessorCount;
+    c.initialized = true;
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_shutdown(void) {
+    ghip::Context& c = ctx();
+    if (!c.initialized) return GRANITE_HIP_OK;
+    (void)hipStreamSynchronize(c.stream);
+    if (c.workspace) (void)hipFree(c.workspace);
+    c.workspace = nullptr;
+    c.workspace_bytes = 0;
+    if (c.own_stream) (void)hipStreamDestroy(c.own_stream);
+    c.own_stream = nullptr;
+    c.stream = nullptr;
+    c.initialized = false;
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_is_initialized(void) { return ctx().initialized ? 1 : 0; }
+
+int granite_hip_get_device_info(granite_hip_device_info* info) {
+    GHIP_REQUIRE_INIT();
+    if (!info) return GRANITE_HIP_ENULL;
+    hipDeviceProp_t prop;
+    GHIP_CHECK(hipGetDeviceProperties(&prop, ctx().device));
+    std::memset(info, 0, sizeof(*info));
+    std::snprintf(info->name, sizeof(info->name), "%s", prop.name);
+    std::snprintf(info->arch, sizeof(info->arch), "%s", prop.gcnArchName);
+    info->total_memory = prop.totalGlobalMem;
+    info->max_buffer_size = prop.totalGlobalMem;
+    info->shared_memory_per_block = prop.sharedMemPerBlock;
+    info->max_threads_per_block = prop.maxThreadsPerBlock;
+    info->wavefront_size = prop.warpSize;
+    info->compute_units = prop.multiProcessorCount;
+    info->clock_khz = prop.clockRate;
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_malloc(void** ptr, size_t bytes, int memory_kind) {
+    GHIP_REQUIRE_INIT();
+    if (!ptr) return GRANITE_HIP_ENULL;
+    *ptr = nullptr;
+    if (bytes == 0) return GRANITE_HIP_EINVAL;
+    hipError_t e;
+    if (memory_kind == GRANITE_HIP_MEM_SHARED)
+        e = hipHostMalloc(ptr, bytes, hipHostMallocDefault);
+    else if (memory_kind == GRANITE_HIP_MEM_DEVICE || memory_kind == GRANITE_HIP_MEM_MANAGED)
+        e = hipMalloc(ptr, bytes);
+    else
+        return GRANITE_HIP_EINVAL;
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *ptr = nullptr;
+        return e == hipErrorOutOfMemory ? GRANITE_HIP_ENOMEM : static_cast<int>(e);
+    }
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_free(void* ptr, int memory_kind) {
+    GHIP_REQUIRE_INIT();
+    if (!ptr) return GRANITE_HIP_OK;
+    if (memory_kind == GRANITE_HIP_MEM_SHARED) GHIP_CHECK(hipHostFree(ptr));
+    else GHIP_CHECK(hipFree(ptr));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    GHIP_REQUIRE_INIT();
+    if (bytes == 0) return GRANITE_HIP_OK;
+    if (!dst || !src) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
+    GHIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    GHIP_REQUIRE_INIT();
+    if (bytes == 0) return GRANITE_HIP_OK;
+    if (!dst || !src) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+    GHIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    GHIP_REQUIRE_INIT();
+    if (bytes == 0) return GRANITE_HIP_OK;
+    if (!dst || !src) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_memset(void* dst, int value, size_t bytes) {
+    GHIP_REQUIRE_INIT();
+    if (bytes == 0) return GRANITE_HIP_OK;
+    if (!dst) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipMemsetAsync(dst, value, bytes, ctx().stream));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_sync(void) {
+    GHIP_REQUIRE_INIT();
+    GHIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_set_stream(void* stream) {
+    GHIP_REQUIRE_INIT();
+    ctx().stream = stream ? static_cast<hipStream_t>(stream) : ctx().own_stream;
+    return GRANITE_HIP_OK;
+}
+
+void* granite_hip_get_stream(void) { return ctx().initialized ? ctx().stream : nullptr; }
+
+int granite_hip_event_create(void** event) {
+    GHIP_REQUIRE_INIT();
+    if (!event) return GRANITE_HIP_ENULL;
+    hipEvent_t e;
+    GHIP_CHECK(hipEventCreate(&e));
+    *event = e;
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_event_destroy(void* event) {
+    GHIP_REQUIRE_INIT();
+    if (!event) return GRANITE_HIP_OK;
+    GHIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_event_record(void* event) {
+    GHIP_REQUIRE_INIT();
+    if (!event) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), ctx().stream));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_event_synchronize(void* event) {
+    GHIP_REQUIRE_INIT();
+    if (!event) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
+    GHIP_REQUIRE_INIT();
+    if (!start || !stop || !ms) return GRANITE_HIP_ENULL;
+    GHIP_CHECK(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start),
+                                   static_cast<hipEvent_t>(stop)));
+    return GRANITE_HIP_OK;
+}
+
+size_t granite_hip_workspace_bytes(void) { return ctx().workspace_bytes; }
+
+// ---- KV append / gather -------------------------------------------------
+
+int granite_hip_kv_cache_append(void* cache_k, void* cache_v, const void* new_k,
+                                const void* new_v, uint32_t num_kv_heads, uint32_t head_dim,
+                                uint32_t current_len, uint32_t new_len, uint32_t max_seq_len) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_kv_append_contig(cache_k, cache_v, new_k, new_v, GRANITE_HIP_F32,
+                                         int64_t(num_kv_heads) * head_dim, head_dim, num_kv_heads,
+                                         head_dim, current_len, new_len, max_seq_len,
+                                         GRANITE_HIP_ROUND_TRUNCATE);
+}
+
+int granite_hip_kv_cache_append_ex(void* cache_k, void* cache_v, const void* new_k,
+                                   const void* new_v, int src_dtype, int64_t src_tok_stride,
+                                   int64_t src_head_stride, uint32_t num_kv_heads,
+                                   uint32_t head_dim, uint32_t current_len, uint32_t new_len,
+                                   uint32_t max_seq_len, int rounding) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_kv_append_contig(cache_k, cache_v, new_k, new_v, src_dtype,
+                                         src_tok_stride, src_head_stride, num_kv_heads, head_dim,
+                                         current_len, new_len, max_seq_len, rounding);
+}
+
+int granite_hip_paged_kv_cache_append(const void* new_k, const void* new_v, void* k_cache,
+                                      void* v_cache, const int32_t* block_table,
+                                      uint32_t num_kv_heads, uint32_t head_dim,
+                                      uint32_t start_pos, uint32_t new_len, uint32_t block_size) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_kv_append_paged(new_k, new_v, GRANITE_HIP_F32, head_dim,
+                                        int64_t(new_len) * head_dim, k_cache, v_cache, block_table,
+                                        num_kv_heads, head_dim, start_pos, new_len, block_size,
+                                        GRANITE_HIP_ROUND_TRUNCATE);
+}
+
+int granite_hip_paged_kv_cache_append_ex(const void* new_k, const void* new_v, int src_dtype,
+                                         int64_t src_tok_stride, int64_t src_head_stride,
+                                         void* k_cache, void* v_cache,
+                                         const int32_t* block_table, uint32_t num_kv_heads,
+                                         uint32_t head_dim, uint32_t start_pos,
+                                         uint32_t new_len, uint32_t block_size, int rounding) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_kv_append_paged(new_k, new_v, src_dtype, src_tok_stride, src_head_stride,
+                                        k_cache, v_cache, block_table, num_kv_heads, head_dim,
+                                        start_pos, new_len, block_size, rounding);
+}
+
+int granite_hip_paged_kv_gather(void* dst_k, void* dst_v, const void* k_cache,
+                                const void* v_cache, const int32_t* block_table,
+                                uint32_t num_kv_heads, uint32_t head_dim, uint32_t len,
+                                uint32_t block_size, uint32_t max_seq_len) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_kv_gather_paged(dst_k, dst_v, k_cache, v_cache, block_table, num_kv_heads,
+                                        head_dim, len, block_size, max_seq_len);
+}
+
+// ---- attention ------------------------------------------------------------
+
+int granite_hip_decode_attention(const granite_hip_decode_args* args) {
+    GHIP_REQUIRE_INIT();
+    if (!args) return GRANITE_HIP_ENULL;
+    return ghip::launch_decode(*args);
+}
+
+int granite_hip_attention(const granite_hip_attention_args* args) {
+    GHIP_REQUIRE_INIT();
+    if (!args) return GRANITE_HIP_ENULL;
+    return ghip::launch_attention(*args);
+}
+
+int granite_hip_build_tree_mask(const int32_t* parent_indices, uint32_t* mask_words,
+                                uint32_t num_nodes) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_tree_mask(parent_indices, mask_words, num_nodes);
+}
+
+int granite_hip_multihead_attention(const void* q, const void* k, const void* v, void* out,
+                                    uint32_t num_heads, uint32_t num_kv_heads, uint32_t seq_q,
+                                    uint32_t seq_kv, uint32_t head_dim, float scale,
+                                    uint32_t max_seq) {
+    GHIP_REQUIRE_INIT();
+    if (max_seq == 0) max_seq = seq_kv;  // metal_compute.mm:2259-2260
+    if (seq_kv == 0 || seq_kv > max_seq) return GRANITE_HIP_EINVAL;
+    if (seq_q == 1) {
+        // Decode: one workgroup set over the contiguous cache, length fixed by the caller.
+        granite_hip_decode_args d{};
+        d.q = q;
+        d.q_dtype = GRANITE_HIP_F32;
+        d.k_cache = k;
+        d.v_cache = v;
+        d.out = out;
+        d.batch_size = 1;
+        d.num_heads = num_heads;
+        d.num_kv_heads = num_kv_heads;
+        d.head_dim = head_dim;
+        d.max_seq = max_seq;
+        d.fixed_seq_len = seq_kv;
+        d.scale = scale;
+        return ghip::launch_decode(d);
+    }
+    granite_hip_attention_args a{};
+    a.q = q;
+    a.q_dtype = GRANITE_HIP_F32;
+    a.q_tok_stride = int64_t(num_heads) * head_dim;
+    a.q_head_stride = head_dim;
+    a.out = out;
+    a.out_dtype = GRANITE_HIP_F32;
+    a.out_tok_stride = a.q_tok_stride;
+    a.out_head_stride = head_dim;
+    a.k_cache = k;
+    a.v_cache = v;
+    a.max_seq = max_seq;
+    a.cache_len = seq_kv;
+    a.mask_mode = GRANITE_HIP_MASK_CAUSAL;
+    a.start_pos = 0;  // the reference passes 0 to its prefill kernel (metal_compute.mm:2352)
+    a.seq_q = seq_q;
+    a.num_heads = num_heads;
+    a.num_kv_heads = num_kv_heads;
+    a.head_dim = head_dim;
+    a.scale = scale;
+    return ghip::launch_attention(a);
+}
+
+int granite_hip_attention_tree(const void* q, const void* k_cache, const void* v_cache,
+                               const void* k_tree, const void* v_tree,
+                               const int32_t* parent_indices, void* out, uint32_t num_heads,
+                               uint32_t num_kv_heads, uint32_t num_nodes, uint32_t cache_len,
+                               uint32_t head_dim, float scale) {
+    GHIP_REQUIRE_INIT();
+    granite_hip_attention_args a{};
+    a.q = q;
+    a.q_dtype = GRANITE_HIP_F32;
+    a.q_tok_stride = head_dim;  // [num_heads, num_nodes, D]
+    a.q_head_stride = int64_t(num_nodes) * head_dim;
+    a.out = out;
+    a.out_dtype = GRANITE_HIP_F32;
+    a.out_tok_stride = head_dim;
+    a.out_head_stride = a.q_head_stride;
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.max_seq = cache_len;
+    a.cache_len = cache_len;
+    a.k_extra = k_tree;
+    a.v_extra = v_tree;
+    a.extra_len = num_nodes;
+    a.parents = parent_indices;
+    a.mask_mode = GRANITE_HIP_MASK_TREE;
+    a.seq_q = num_nodes;
+    a.num_heads = num_heads;
+    a.num_kv_heads = num_kv_heads;
+    a.head_dim = head_dim;
+    a.scale = scale;
+    return ghip::launch_attention(a);
+}
+
+int granite_hip_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
+                                       const int32_t* block_table, void* out,
+                                       uint32_t num_heads, uint32_t num_kv_heads,
+                                       uint32_t seq_len, uint32_t head_dim,
+                                       uint32_t block_size, float scale) {
+    GHIP_REQUIRE_INIT();
+    if (!block_table) return GRANITE_HIP_ENULL;
+    if (seq_len == 0 || block_size == 0) return GRANITE_HIP_EINVAL;
+    granite_hip_decode_args d{};
+    d.q = q;
+    d.q_dtype = GRANITE_HIP_F32;
+    d.k_cache = k_cache;
+    d.v_cache = v_cache;
+    d.block_tables = block_table;
+    d.out = out;
+    d.batch_size = 1;
+    d.num_heads = num_heads;
+    d.num_kv_heads = num_kv_heads;
+    d.head_dim = head_dim;
+    d.block_size = block_size;
+    d.max_blocks_per_seq = (seq_len + block_size - 1) / block_size;
+    d.fixed_seq_len = seq_len;
+    d.scale = scale;
+    return ghip::launch_decode(d);
+}
+
+int granite_hip_batched_paged_attention_decode(const void* q, const void* k_cache,
+                                               const void* v_cache,
+                                               const int32_t* block_tables,
+                                               const int32_t* seq_lens, void* out,
+                                               uint32_t batch_size, uint32_t num_heads,
+                                               uint32_t num_kv_heads, uint32_t head_dim,
+                                               uint32_t block_size,
+                                               uint32_t max_blocks_per_seq, float scale) {
+    GHIP_REQUIRE_INIT();
+    if (!block_tables || !seq_lens) return GRANITE_HIP_ENULL;
+    granite_hip_decode_args d{};
+    d.q = q;
+    d.q_dtype = GRANITE_HIP_F32;
+    d.k_cache = k_cache;
+    d.v_cache = v_cache;
+    d.block_tables = block_tables;
+    d.seq_lens = seq_lens;
+    d.out = out;
+    d.batch_size = batch_size;
+    d.num_heads = num_heads;
+    d.num_kv_heads = num_kv_heads;
+    d.head_dim = head_dim;
+    d.block_size = block_size;
+    d.max_blocks_per_seq = max_blocks_per_seq;
+    d.scale = scale;
+    return ghip::launch_decode(d);
+}
+
+}  // extern "C"

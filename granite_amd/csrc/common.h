@@ -1,0 +1,108 @@
+// Shared declarations of the gfx950 attention library: launch-side context,
+// error helpers and the small device utilities every kernel file uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "granite_hip.h"
+
+namespace ghip {
+
+constexpr int kHeadDim = 128;  // the attention kernels are specialised for D = 128
+constexpr int kWave = 64;      // CDNA wavefront
+
+// Process-wide launch context (one in-order stream, one scratch buffer).
+struct Context {
+    bool initialized = false;
+    int device = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;  // the stream launches go to
+    void* workspace = nullptr;     // split-K partials, tree masks
+    size_t workspace_bytes = 0;
+    int compute_units = 0;
+};
+
+Context& ctx();
+
+// Grows the scratch buffer to at least `bytes` (stream-ordered with respect
+// to earlier launches: the old buffer is released only after a sync).
+int ensure_workspace(size_t bytes);
+
+#define GHIP_CHECK(expr)                               \
+    do {                                               \
+        hipError_t _e = (expr);                        \
+        if (_e != hipSuccess) return static_cast<int>(_e); \
+    } while (0)
+
+#define GHIP_REQUIRE_INIT()                                   \
+    do {                                                      \
+        if (!::ghip::ctx().initialized) return GRANITE_HIP_ENOTINIT; \
+    } while (0)
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? GRANITE_HIP_OK : static_cast<int>(e);
+}
+
+// ---- launchers implemented in the kernel files -------------------------
+int launch_kv_append_contig(void* cache_k, void* cache_v, const void* new_k, const void* new_v,
+                            int src_dtype, int64_t src_tok_stride, int64_t src_head_stride,
+                            uint32_t num_kv_heads, uint32_t head_dim, uint32_t current_len,
+                            uint32_t new_len, uint32_t max_seq_len, int rounding);
+int launch_kv_append_paged(const void* new_k, const void* new_v, int src_dtype,
+                           int64_t src_tok_stride, int64_t src_head_stride, void* k_cache,
+                           void* v_cache, const int32_t* block_table, uint32_t num_kv_heads,
+                           uint32_t head_dim, uint32_t start_pos, uint32_t new_len,
+                           uint32_t block_size, int rounding);
+int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const void* v_cache,
+                           const int32_t* block_table, uint32_t num_kv_heads, uint32_t head_dim,
+                           uint32_t len, uint32_t block_size, uint32_t max_seq_len);
+int launch_decode(const granite_hip_decode_args& a);
+int launch_attention(const granite_hip_attention_args& a);
+int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes);
+
+// ---- device helpers ------------------------------------------------------
+#if defined(__HIPCC__)
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+// Granite's truncating float->half (src/llm/math_ops.cpp:45-54), bit for bit.
+__device__ __forceinline__ uint16_t f32_to_f16_truncate(float f) {
+    uint32_t bits = __float_as_uint(f);
+    uint32_t sign = (bits >> 16) & 0x8000u;
+    int32_t e = static_cast<int32_t>((bits >> 23) & 0xFFu) - 127 + 15;
+    uint32_t mant = (bits >> 13) & 0x3FFu;
+    if (e <= 0) return static_cast<uint16_t>(sign);
+    if (e >= 31) return static_cast<uint16_t>(sign | 0x7C00u);
+    return static_cast<uint16_t>(sign | (static_cast<uint32_t>(e) << 10) | mant);
+}
+
+// Round-to-nearest-even float->half, what Metal's half(x) does.
+__device__ __forceinline__ uint16_t f32_to_f16_nearest(float f) {
+    _Float16 h = static_cast<_Float16>(f);
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    half2v v;
+    v.x = static_cast<_Float16>(lo);
+    v.y = static_cast<_Float16>(hi);
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float wave_shfl_xor(float v, int mask) {
+    return __shfl_xor(v, mask, kWave);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace ghip

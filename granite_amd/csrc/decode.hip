@@ -1,0 +1,374 @@
+// Paged / contiguous KV decode attention for gfx950: split-K over the context,
+// MFMA tiles fed straight from global memory, log-sum-exp merge.
+//
+// Stands in for the reference decode kernels
+//   flash_attention_decode_d128            metal_shaders_attention.h:2982-3177
+//   paged_flash_attention_decode_d128      metal_shaders_attention.h:3660-3847
+//   batched_paged_attention_decode         metal_shaders_attention.h:2186-2304
+// with the arithmetic of the CPU path (src/llm/transformer.mm:1779-1840): fp32
+// scores, softmax without epsilon, GQA head h reads KV head h / G.
+//
+// Work split.  grid = (chunks, kv_heads * q_groups, sequences).  A workgroup
+// of 4 waves owns one (sequence, KV head, chunk of `chunk_tokens` tokens) and
+// all G query heads of that KV head, so every K/V byte is fetched once.  Each
+// wave walks 32-token tiles of the chunk (tile index = wave, wave+4, ...):
+//
+//   S^T[tok, q]  = K[tok, :] . Q[q, :]        8 x v_mfma_f32_16x16x32_f16
+//   online softmax in the MFMA result layout  (a lane owns ONE query head and
+//                                              8 tokens: no cross-lane traffic
+//                                              except two shuffles for the max)
+//   O^T[d, q]   += V^T[d, tok] . P^T[tok, q]  8 x v_mfma_f32_16x16x32_f16
+//
+// Operand layouts are chosen so that nothing goes through LDS:
+//   * K rows are the MFMA A operand as they lie in memory: lane (m = lane%16,
+//     g = lane/16) loads 16 bytes of token m at d = 32*step + 8*g.
+//   * the token order inside the PV contraction is permuted (tau below) so the
+//     probabilities a lane holds after the first MFMA are exactly the B
+//     operand of the second;
+//   * V rows are loaded 16 bytes per lane (token tau(g, j), d = 8m..8m+7) and
+//     turned into the A operand by an 8x8 in-register transpose made of
+//     v_perm_b32; output row m of d-tile t stands for d = 8m + t, which makes
+//     each lane end up with 32 consecutive output floats.
+// The four waves' (m, l, O) are merged through LDS, written as one partial per
+// (sequence, query head, chunk), and a second kernel merges the chunks.
+//
+// Algorithmic HBM bytes per token of context: 2 (K,V) * num_kv_heads * 128 * 2.
+#include "common.h"
+
+namespace ghip {
+namespace {
+
+constexpr int kTile = 32;         // tokens per wave step
+constexpr int kWavesPerWG = 4;
+constexpr float kNegBig = -1.0e30f;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct DecodeParams {
+    const void* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    const int32_t* tables;
+    const int32_t* seq_lens;
+    float* part_o;   // [B, Hq, max_chunks, D]
+    float* part_ml;  // [B, Hq, max_chunks, 2]
+    float* out;
+    float* lse;
+    uint32_t batch, num_heads, num_kv_heads, group, q_groups;
+    uint32_t block_size, max_blocks;
+    int bs_shift;  // log2(block_size) or -1
+    int64_t tok_stride, head_stride;
+    uint32_t max_tokens;  // bound on any sequence length
+    uint32_t chunk_tokens, max_chunks;
+    float scale_log2;
+};
+
+__device__ __forceinline__ size_t phys_row(const DecodeParams& p, const int32_t* table,
+                                           uint32_t tok) {
+    if (!table) return tok;
+    uint32_t blk, off;
+    if (p.bs_shift >= 0) {
+        blk = tok >> p.bs_shift;
+        off = tok & (p.block_size - 1);
+    } else {
+        blk = tok / p.block_size;
+        off = tok - blk * p.block_size;
+    }
+    return size_t(table[blk]) * p.block_size + off;
+}
+
+// Token handled by slot j (0..7) of lane group g in the PV contraction.
+__device__ __forceinline__ uint32_t tau(uint32_t g, uint32_t j) {
+    return j < 4 ? 4 * g + j : 16 + 4 * g + (j - 4);
+}
+
+__device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
+
+template <bool kQF32>
+__global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(DecodeParams p) {
+    const uint32_t chunk = blockIdx.x;
+    const uint32_t kvh = blockIdx.y / p.q_groups;
+    const uint32_t qg = blockIdx.y % p.q_groups;
+    const uint32_t b = blockIdx.z;
+
+    uint32_t len = p.seq_lens ? uint32_t(max(p.seq_lens[b], 0)) : p.max_tokens;
+    len = min(len, p.max_tokens);
+    const uint32_t chunk_start = chunk * p.chunk_tokens;
+    if (chunk_start >= len) return;
+    const uint32_t chunk_end = min(len, chunk_start + p.chunk_tokens);
+    const uint32_t n_tiles = (chunk_end - chunk_start + kTile - 1) / kTile;
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t n = lane & 15;  // MFMA column: query head within the group / row index m
+    const uint32_t g = lane >> 4;  // MFMA k-group
+
+    const uint32_t q_in_group = qg * 16 + n;  // query head index inside the GQA group
+    const bool q_valid = q_in_group < p.group;
+    const uint32_t qh = kvh * p.group + (q_valid ? q_in_group : 0);
+
+    const int32_t* table = p.tables ? p.tables + size_t(b) * p.max_blocks : nullptr;
+    const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride;
+    const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride;
+
+    // ---- Q as MFMA B operand: lane (n, g), step s holds Q[qh][32s + 8g .. +7]
+    half8 bq[4];
+    half8 bq_lo[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        half8 hi = {0, 0, 0, 0, 0, 0, 0, 0};
+        half8 lo = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (q_valid) {
+            const size_t off = (size_t(b) * p.num_heads + qh) * kHeadDim + 32 * s + 8 * g;
+            if constexpr (kQF32) {
+                const float* qp = static_cast<const float*>(p.q) + off;
+                float4v x0 = *reinterpret_cast<const float4v*>(qp);
+                float4v x1 = *reinterpret_cast<const float4v*>(qp + 4);
+                float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    _Float16 h = static_cast<_Float16>(x[i]);
+                    hi[i] = h;
+                    lo[i] = static_cast<_Float16>(x[i] - static_cast<float>(h));
+                }
+            } else {
+                hi = as_half8(*reinterpret_cast<const uint4v*>(
+                    static_cast<const uint16_t*>(p.q) + off));
+            }
+        }
+        bq[s] = hi;
+        bq_lo[s] = lo;
+    }
+
+    float m_run = kNegBig;  // running max (log2 domain), identical in the 4 lanes of a column
+    float l_run = 0.0f;     // running sum, lane-partial (summed over g at the end)
+    float4v acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[t] = float4v{0, 0, 0, 0};
+
+    for (uint32_t tile = wave; tile < n_tiles; tile += kWavesPerWG) {
+        const uint32_t tok0 = chunk_start + tile * kTile;
+
+        // ---- K tile: two 16-token sub-tiles, 4 k-steps each
+        half8 ka[2][4];
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            uint32_t tok = min(tok0 + 16 * sub + n, len - 1);
+            const uint16_t* kp = kbase + phys_row(p, table, tok) * p.tok_stride + 8 * g;
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                ka[sub][s] = as_half8(*reinterpret_cast<const uint4v*>(kp + 32 * s));
+        }
+        // ---- V tile: 8 token rows per lane, 16 bytes each
+        uint4v vr[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t tok = min(tok0 + tau(g, j), len - 1);
+            const uint16_t* vp = vbase + phys_row(p, table, tok) * p.tok_stride + 8 * n;
+            vr[j] = *reinterpret_cast<const uint4v*>(vp);
+        }
+
+        // ---- S^T = K Q^T
+        float4v c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[0][s], bq[s], c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[1][s], bq[s], c1, 0, 0, 0);
+            if constexpr (kQF32) {
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[0][s], bq_lo[s], c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[1][s], bq_lo[s], c1, 0, 0, 0);
+            }
+        }
+
+        // ---- online softmax; lane (n, g) holds tokens 4g+r and 16+4g+r of column n
+        float s[8];
+        float mloc = kNegBig;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float a = c0[r] * p.scale_log2;
+            float bsc = c1[r] * p.scale_log2;
+            if (tok0 + 4 * g + r >= chunk_end) a = -INFINITY;
+            if (tok0 + 16 + 4 * g + r >= chunk_end) bsc = -INFINITY;
+            s[r] = a;
+            s[4 + r] = bsc;
+            mloc = fmaxf(mloc, fmaxf(a, bsc));
+        }
+        mloc = fmaxf(mloc, wave_shfl_xor(mloc, 16));
+        mloc = fmaxf(mloc, wave_shfl_xor(mloc, 32));
+        const float m_new = fmaxf(m_run, mloc);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.0f;
+        float pj[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            pj[j] = fast_exp2(s[j] - m_new);
+            psum += pj[j];
+        }
+        l_run = l_run * alpha + psum;
+        uint4v bpw;
+        bpw.x = pack_f16x2(pj[0], pj[1]);
+        bpw.y = pack_f16x2(pj[2], pj[3]);
+        bpw.z = pack_f16x2(pj[4], pj[5]);
+        bpw.w = pack_f16x2(pj[6], pj[7]);
+        const half8 bp = as_half8(bpw);
+
+        // ---- O^T += V^T P^T : 8 d-tiles, A operand by in-register transpose
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+            uint4v aw;
+            aw.x = __builtin_amdgcn_perm(vr[1][t >> 1], vr[0][t >> 1], sel);
+            aw.y = __builtin_amdgcn_perm(vr[3][t >> 1], vr[2][t >> 1], sel);
+            aw.z = __builtin_amdgcn_perm(vr[5][t >> 1], vr[4][t >> 1], sel);
+            aw.w = __builtin_amdgcn_perm(vr[7][t >> 1], vr[6][t >> 1], sel);
+            float4v cin = acc[t] * alpha;
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(aw), bp, cin, 0, 0, 0);
+        }
+    }
+
+    // ---- reduce the lane-partial sums over the 4 k-groups
+    l_run += wave_shfl_xor(l_run, 16);
+    l_run += wave_shfl_xor(l_run, 32);
+
+    // ---- merge the 4 waves through LDS
+    constexpr int kRowPad = kHeadDim + 4;
+    __shared__ float s_o[kWavesPerWG][16][kRowPad];
+    __shared__ float s_m[kWavesPerWG][16];
+    __shared__ float s_l[kWavesPerWG][16];
+    if (g == 0) {
+        s_m[wave][n] = m_run;
+        s_l[wave][n] = l_run;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) s_o[wave][n][32 * g + 8 * r + t] = acc[t][r];
+    __syncthreads();
+
+    const uint32_t rows = min(p.group - qg * 16, 16u);
+    for (uint32_t i = threadIdx.x; i < rows * kHeadDim; i += blockDim.x) {
+        const uint32_t row = i / kHeadDim, d = i % kHeadDim;
+        float mx = s_m[0][row];
+#pragma unroll
+        for (int w = 1; w < kWavesPerWG; w++) mx = fmaxf(mx, s_m[w][row]);
+        float o = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerWG; w++) {
+            const float f = fast_exp2(s_m[w][row] - mx);
+            o += s_o[w][row][d] * f;
+            l += s_l[w][row] * f;
+        }
+        const size_t head = size_t(b) * p.num_heads + kvh * p.group + qg * 16 + row;
+        const size_t slot = head * p.max_chunks + chunk;
+        p.part_o[slot * kHeadDim + d] = o;
+        if (d == 0) {
+            p.part_ml[slot * 2 + 0] = mx;
+            p.part_ml[slot * 2 + 1] = l;
+        }
+    }
+}
+
+// Merges the per-chunk partials of one (sequence, query head):
+//   M = max_c m_c,  L = sum_c l_c 2^(m_c - M),  out = sum_c O_c 2^(m_c - M) / L,
+//   lse = (M + log2 L) ln 2.
+__global__ void __launch_bounds__(kHeadDim) decode_merge_kernel(DecodeParams p) {
+    const uint32_t qh = blockIdx.x;
+    const uint32_t b = blockIdx.y;
+    uint32_t len = p.seq_lens ? uint32_t(max(p.seq_lens[b], 0)) : p.max_tokens;
+    len = min(len, p.max_tokens);
+    if (len == 0) return;  // untouched, as the reference kernel does for empty sequences
+    const uint32_t n_chunks = (len + p.chunk_tokens - 1) / p.chunk_tokens;
+    const size_t head = size_t(b) * p.num_heads + qh;
+    const float* ml = p.part_ml + head * p.max_chunks * 2;
+    const float* po = p.part_o + head * p.max_chunks * kHeadDim;
+    const uint32_t d = threadIdx.x;
+
+    float mx = kNegBig;
+    for (uint32_t c = 0; c < n_chunks; c++) mx = fmaxf(mx, ml[2 * c]);
+    float o = 0.0f, l = 0.0f;
+    for (uint32_t c = 0; c < n_chunks; c++) {
+        const float f = fast_exp2(ml[2 * c] - mx);
+        l += ml[2 * c + 1] * f;
+        o += po[size_t(c) * kHeadDim + d] * f;
+    }
+    p.out[head * kHeadDim + d] = o / l;
+    if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
+}
+
+}  // namespace
+
+static size_t g_decode_workspace = 0;
+
+int launch_decode(const granite_hip_decode_args& a) {
+    if (!a.q || !a.k_cache || !a.v_cache || !a.out) return GRANITE_HIP_ENULL;
+    if (a.head_dim != kHeadDim) return GRANITE_HIP_EINVAL;
+    if (a.num_heads == 0 || a.num_kv_heads == 0 || a.num_heads % a.num_kv_heads != 0)
+        return GRANITE_HIP_EINVAL;
+    if (a.q_dtype != GRANITE_HIP_F32 && a.q_dtype != GRANITE_HIP_F16) return GRANITE_HIP_EINVAL;
+    if (a.batch_size == 0) return GRANITE_HIP_OK;
+
+    DecodeParams p{};
+    p.q = a.q;
+    p.k = static_cast<const uint16_t*>(a.k_cache);
+    p.v = static_cast<const uint16_t*>(a.v_cache);
+    p.tables = a.block_tables;
+    p.seq_lens = a.seq_lens;
+    p.out = static_cast<float*>(a.out);
+    p.lse = a.lse;
+    p.batch = a.batch_size;
+    p.num_heads = a.num_heads;
+    p.num_kv_heads = a.num_kv_heads;
+    p.group = a.num_heads / a.num_kv_heads;
+    p.q_groups = (p.group + 15) / 16;
+    if (a.block_tables) {
+        if (a.block_size == 0 || a.max_blocks_per_seq == 0) return GRANITE_HIP_EINVAL;
+        p.block_size = a.block_size;
+        p.max_blocks = a.max_blocks_per_seq;
+        p.bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
+        p.tok_stride = int64_t(a.num_kv_heads) * kHeadDim;
+        p.head_stride = kHeadDim;
+        const uint64_t mt = uint64_t(a.block_size) * a.max_blocks_per_seq;
+        if (mt >= (1ull << 31)) return GRANITE_HIP_EINVAL;
+        p.max_tokens = static_cast<uint32_t>(mt);
+    } else {
+        if (a.batch_size != 1 || a.max_seq == 0) return GRANITE_HIP_EINVAL;
+        p.block_size = 1;
+        p.max_blocks = 0;
+        p.bs_shift = 0;
+        p.tok_stride = kHeadDim;
+        p.head_stride = int64_t(a.max_seq) * kHeadDim;
+        p.max_tokens = a.max_seq;
+    }
+    if (!a.seq_lens) {
+        if (a.fixed_seq_len == 0 || a.fixed_seq_len > p.max_tokens) return GRANITE_HIP_EINVAL;
+        p.max_tokens = a.fixed_seq_len;
+    }
+    p.chunk_tokens = a.chunk_tokens ? a.chunk_tokens : 256;
+    if (p.chunk_tokens % kTile != 0) return GRANITE_HIP_EINVAL;
+    p.max_chunks = (p.max_tokens + p.chunk_tokens - 1) / p.chunk_tokens;
+    p.scale_log2 = a.scale * kLog2e;
+
+    const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;
+    const size_t need = slots * (kHeadDim + 2) * sizeof(float);
+    int rc = ensure_workspace(need);
+    if (rc != GRANITE_HIP_OK) return rc;
+    p.part_o = static_cast<float*>(ctx().workspace);
+    p.part_ml = p.part_o + slots * kHeadDim;
+    g_decode_workspace = need;
+
+    if (p.max_chunks > 65535u * 32 || p.batch > 65535u) return GRANITE_HIP_EINVAL;
+    dim3 grid(p.max_chunks, p.num_kv_heads * p.q_groups, p.batch);
+    dim3 block(kWavesPerWG * kWave);
+    hipStream_t st = ctx().stream;
+    if (a.q_dtype == GRANITE_HIP_F32)
+        decode_splitk_kernel<true><<<grid, block, 0, st>>>(p);
+    else
+        decode_splitk_kernel<false><<<grid, block, 0, st>>>(p);
+    rc = launch_status();
+    if (rc != GRANITE_HIP_OK) return rc;
+    decode_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(kHeadDim), 0, st>>>(p);
+    return launch_status();
+}
+
+}  // namespace ghip

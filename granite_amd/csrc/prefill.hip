@@ -1,0 +1,453 @@
+// Causal GQA flash-attention prefill, chunked prefill over a paged cache and
+// tree-masked attention for gfx950 (MFMA, K/V tiles staged in LDS).
+//
+// Stands in for
+//   flash_attention_prefill     src/backend/metal/kernels/metal_shaders_attention.h:1447-1660
+//   attention_tree_f16kv        metal_shaders_attention.h:1677-1865
+// and follows the arithmetic of the CPU path they are checked against:
+//   TransformerModel::attention       src/llm/transformer.mm:1779-1840
+//   TransformerModel::attention_tree  src/llm/transformer.mm:2044-2126
+// (fp32 scores and softmax, no epsilon, key k visible iff k <= start_pos + q;
+// tree: cache keys visible, tree key j visible iff j is q or an ancestor).
+//
+// Structure.  grid = (query tiles of 128 rows, query heads); 4 waves, each
+// owning 32 query rows.  Keys are walked in tiles of 64: the workgroup copies
+// the K tile (as is) and the V tile (transposed, token order permuted) into
+// LDS, then every wave computes, with v_mfma_f32_32x32x16_f16,
+//
+//   S^T[key, q]  = K[key, :] . Q[q, :]          (A = K from LDS, B = Q in VGPRs)
+//   online softmax in the result layout: a lane owns one query row and 32 of
+//   the 64 keys, so max/sum are in-lane plus one cross-half shuffle
+//   O^T[d, q]   += V^T[d, key] . P^T[key, q]    (A = V^T from LDS, B = P in VGPRs)
+//
+// Computing the transposed products makes the softmax output of the first
+// MFMA land exactly in the B-operand layout of the second once the keys of
+// each 16-key group are stored in LDS in the order 8g + 4a + b for key
+// 8a + 4g + b (a, g in {0,1}, b in 0..3).
+//
+// The next tile is fetched from global memory into registers while the
+// current one is being multiplied (one LDS buffer, two barriers per tile).
+//
+// Algorithmic work: 4 * D flops per visible (query, key) pair.
+#include "common.h"
+
+namespace ghip {
+namespace {
+
+constexpr int kBM = 128;       // query rows per workgroup
+constexpr int kBN = 64;        // keys per tile
+constexpr int kThreads = 256;  // 4 waves
+constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
+constexpr int kVPitch = kBN + 8;       // halves per V^T row in LDS
+constexpr float kNegBig = -1.0e30f;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct AttnParams {
+    const void* q;
+    void* out;
+    float* lse;
+    int64_t q_tok_stride, q_head_stride, out_tok_stride, out_head_stride;
+    const uint16_t* k;
+    const uint16_t* v;
+    const int32_t* table;
+    uint32_t block_size;
+    int bs_shift;
+    int64_t a_tok_stride, a_head_stride;
+    uint32_t cache_len;
+    const uint16_t* k_extra;
+    const uint16_t* v_extra;
+    uint32_t extra_len;
+    const uint32_t* tree_mask;
+    uint32_t mask_words;
+    int mask_mode;
+    uint32_t start_pos, seq_q, num_heads, group;
+    float scale_log2;
+};
+
+__device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
+
+__device__ __forceinline__ size_t phys_row(const AttnParams& p, uint32_t tok) {
+    if (!p.table) return tok;
+    uint32_t blk, off;
+    if (p.bs_shift >= 0) {
+        blk = tok >> p.bs_shift;
+        off = tok & (p.block_size - 1);
+    } else {
+        blk = tok / p.block_size;
+        off = tok - blk * p.block_size;
+    }
+    return size_t(p.table[blk]) * p.block_size + off;
+}
+
+// Row pointer (head kvh) of key `idx` of segment A (cache) or B (extra).
+__device__ __forceinline__ const uint16_t* key_row(const AttnParams& p, const uint16_t* base_a,
+                                                   const uint16_t* base_b, bool seg_b,
+                                                   uint32_t idx) {
+    if (seg_b) return base_b + size_t(idx) * kHeadDim;
+    return base_a + phys_row(p, idx) * p.a_tok_stride;
+}
+
+template <bool kQF32, bool kOutF32>
+__global__ void __launch_bounds__(kThreads) attention_tiles_kernel(AttnParams p) {
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[kBN * kKPitch];
+    __shared__ __attribute__((aligned(16))) uint16_t s_vt[kHeadDim * kVPitch];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t n = lane & 31;  // query row inside the wave / MFMA row index m
+    const uint32_t g = lane >> 5;  // MFMA k-group (0/1)
+
+    // heavy (late) query tiles first so the causal tail is short
+    const uint32_t q_tile = gridDim.x - 1 - blockIdx.x;
+    const uint32_t head = blockIdx.y;
+    const uint32_t kvh = head / p.group;
+    const uint32_t q0_wg = q_tile * kBM;
+    const uint32_t q0 = q0_wg + 32 * wave;
+    const uint32_t q_row = q0 + n;
+    const bool wave_active = q0 < p.seq_q;
+    const uint32_t q_ld = min(q_row, p.seq_q - 1);
+
+    // ---- keys this workgroup has to visit
+    uint32_t len_a = p.cache_len;
+    if (p.mask_mode == GRANITE_HIP_MASK_CAUSAL) {
+        const uint32_t q_last = min(q0_wg + kBM, p.seq_q) - 1;
+        len_a = min(len_a, p.start_pos + q_last + 1);
+    }
+    const uint32_t len_b = p.extra_len;
+    const uint32_t tiles_a = (len_a + kBN - 1) / kBN;
+    const uint32_t tiles_b = (len_b + kBN - 1) / kBN;
+    const uint32_t n_tiles = tiles_a + tiles_b;
+
+    const uint16_t* ka_base = p.k + size_t(kvh) * p.a_head_stride;
+    const uint16_t* va_base = p.v + size_t(kvh) * p.a_head_stride;
+    const uint16_t* kb_base = p.k_extra ? p.k_extra + size_t(kvh) * len_b * kHeadDim : nullptr;
+    const uint16_t* vb_base = p.v_extra ? p.v_extra + size_t(kvh) * len_b * kHeadDim : nullptr;
+
+    // ---- Q^T as B operand: lane (n, g), step s holds Q[q][16 s + 8 g .. +7]
+    half8 bq[8];
+    half8 bq_lo[kQF32 ? 8 : 1];
+    {
+        const int64_t qoff = int64_t(q_ld) * p.q_tok_stride + int64_t(head) * p.q_head_stride;
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            if constexpr (kQF32) {
+                const float* qp = static_cast<const float*>(p.q) + qoff + 16 * s + 8 * g;
+                float4v x0 = *reinterpret_cast<const float4v*>(qp);
+                float4v x1 = *reinterpret_cast<const float4v*>(qp + 4);
+                float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                half8 hi, lo;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    _Float16 h = static_cast<_Float16>(x[i]);
+                    hi[i] = h;
+                    lo[i] = static_cast<_Float16>(x[i] - static_cast<float>(h));
+                }
+                bq[s] = hi;
+                bq_lo[s] = lo;
+            } else {
+                const uint16_t* qp = static_cast<const uint16_t*>(p.q) + qoff + 16 * s + 8 * g;
+                bq[s] = as_half8(*reinterpret_cast<const uint4v*>(qp));
+            }
+        }
+    }
+
+    // tree mask row of this lane's query (tree mode keeps <= 2 words in registers
+    // per tile; rows are read from global memory per tile)
+    const uint32_t* mask_row =
+        p.tree_mask ? p.tree_mask + size_t(min(q_row, p.extra_len - 1)) * p.mask_words : nullptr;
+
+    float m_run = kNegBig;
+    float l_run = 0.0f;
+    float16v oacc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[t][r] = 0.0f;
+
+    // ---- global -> register staging of one K/V tile
+    const uint32_t ld_chunk = tid & 15;  // 16-byte column of the 256-byte row
+    const uint32_t ld_row = tid >> 4;    // 0..15
+    uint4v kreg[4], vreg[4];
+
+    auto load_tile = [&](uint32_t it) {
+        const bool seg_b = it >= tiles_a;
+        const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
+        const uint32_t seg_len = seg_b ? len_b : len_a;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t kk = min(key0 + ld_row + 16 * i, seg_len - 1);
+            kreg[i] = *reinterpret_cast<const uint4v*>(key_row(p, ka_base, kb_base, seg_b, kk) +
+                                                       8 * ld_chunk);
+            const uint32_t vk = min(key0 + 4 * ld_row + i, seg_len - 1);
+            vreg[i] = *reinterpret_cast<const uint4v*>(key_row(p, va_base, vb_base, seg_b, vk) +
+                                                       8 * ld_chunk);
+        }
+    };
+
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            *reinterpret_cast<uint4v*>(&s_k[(ld_row + 16 * i) * kKPitch + 8 * ld_chunk]) = kreg[i];
+        // V: 4 keys x 8 d  ->  8 rows (d) of 4 keys; column = permuted key position
+        const uint32_t kq = ld_row;  // key quad 0..15 : keys 4kq .. 4kq+3
+        const uint32_t col = 16 * (kq >> 2) + 8 * (kq & 1) + 4 * ((kq >> 1) & 1);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+            uint2v w;
+            w.x = __builtin_amdgcn_perm(vreg[1][t >> 1], vreg[0][t >> 1], sel);
+            w.y = __builtin_amdgcn_perm(vreg[3][t >> 1], vreg[2][t >> 1], sel);
+            *reinterpret_cast<uint2v*>(&s_vt[(8 * ld_chunk + t) * kVPitch + col]) = w;
+        }
+    };
+
+    if (n_tiles > 0) load_tile(0);
+
+    for (uint32_t it = 0; it < n_tiles; it++) {
+        __syncthreads();
+        store_tile();
+        __syncthreads();
+        if (it + 1 < n_tiles) load_tile(it + 1);
+
+        const bool seg_b = it >= tiles_a;
+        const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
+        const uint32_t seg_len = seg_b ? len_b : len_a;
+
+        bool compute = wave_active;
+        if (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !seg_b) {
+            const uint32_t q_last_wave = min(q0 + 32, p.seq_q) - 1;
+            if (key0 > p.start_pos + q_last_wave) compute = false;
+        }
+        if (!compute) continue;
+
+        // ---- S^T for the two 32-key sub-tiles
+        float16v sacc[2];
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) sacc[sub][r] = 0.0f;
+            const uint16_t* krow = &s_k[(32 * sub + n) * kKPitch + 8 * g];
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const half8 a = as_half8(*reinterpret_cast<const uint4v*>(krow + 16 * s));
+                sacc[sub] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[s], sacc[sub], 0, 0, 0);
+                if constexpr (kQF32)
+                    sacc[sub] =
+                        __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[s], sacc[sub], 0, 0, 0);
+            }
+        }
+
+        // ---- masks (only on tiles that need them)
+        const bool partial = key0 + kBN > seg_len;
+        const bool diagonal = p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !seg_b &&
+                              key0 + kBN - 1 > p.start_pos + q0;
+        const bool tree = p.mask_mode == GRANITE_HIP_MASK_TREE && seg_b;
+        if (partial || diagonal || tree) {
+            uint32_t mw0 = 0xFFFFFFFFu, mw1 = 0xFFFFFFFFu;
+            if (tree) {
+                const uint32_t w = key0 >> 5;
+                mw0 = w < p.mask_words ? mask_row[w] : 0u;
+                mw1 = w + 1 < p.mask_words ? mask_row[w + 1] : 0u;
+            }
+            const uint32_t limit = diagonal ? min(seg_len, p.start_pos + q_row + 1) : seg_len;
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++) {
+                const uint32_t mw = sub ? mw1 : mw0;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t kin = 8 * (r >> 2) + 4 * g + (r & 3);  // key inside sub-tile
+                    const bool vis = (key0 + 32 * sub + kin < limit) && ((mw >> kin) & 1u);
+                    if (!vis) sacc[sub][r] = -INFINITY;
+                }
+            }
+        }
+
+        // ---- online softmax (raw scores; the scale is folded into the exponent)
+        float mraw = -INFINITY;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[sub][r]);
+        mraw = fmaxf(mraw, wave_shfl_xor(mraw, 32));
+        const float m_new = fmaxf(m_run, mraw * p.scale_log2);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.0f;
+        half8 bp[2][2];
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                float pe[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    pe[j] = fast_exp2(__builtin_fmaf(sacc[sub][8 * u + j], p.scale_log2, -m_new));
+                    psum += pe[j];
+                }
+                uint4v w;
+                w.x = pack_f16x2(pe[0], pe[1]);
+                w.y = pack_f16x2(pe[2], pe[3]);
+                w.z = pack_f16x2(pe[4], pe[5]);
+                w.w = pack_f16x2(pe[6], pe[7]);
+                bp[sub][u] = as_half8(w);
+            }
+        l_run = l_run * alpha + psum;
+
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
+            const uint16_t* vrow = &s_vt[(32 * t + n) * kVPitch + 8 * g];
+#pragma unroll
+            for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const half8 a =
+                        as_half8(*reinterpret_cast<const uint4v*>(vrow + 32 * sub + 16 * u));
+                    oacc[t] =
+                        __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp[sub][u], oacc[t], 0, 0, 0);
+                }
+        }
+    }
+
+    if (!wave_active) return;
+    l_run += wave_shfl_xor(l_run, 32);
+    if (q_row >= p.seq_q) return;
+    const float inv_l = 1.0f / l_run;
+    const int64_t ooff = int64_t(q_row) * p.out_tok_stride + int64_t(head) * p.out_head_stride;
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const uint32_t d = 32 * t + 8 * a + 4 * g;
+            const float x0 = oacc[t][4 * a + 0] * inv_l, x1 = oacc[t][4 * a + 1] * inv_l;
+            const float x2 = oacc[t][4 * a + 2] * inv_l, x3 = oacc[t][4 * a + 3] * inv_l;
+            if constexpr (kOutF32) {
+                *reinterpret_cast<float4v*>(static_cast<float*>(p.out) + ooff + d) =
+                    float4v{x0, x1, x2, x3};
+            } else {
+                uint2v w;
+                w.x = pack_f16x2(x0, x1);
+                w.y = pack_f16x2(x2, x3);
+                *reinterpret_cast<uint2v*>(static_cast<uint16_t*>(p.out) + ooff + d) = w;
+            }
+        }
+    if (p.lse && g == 0)
+        p.lse[size_t(head) * p.seq_q + q_row] = (m_run + __builtin_amdgcn_logf(l_run)) * kLn2;
+}
+
+// One thread per node: set own bit, then walk parent pointers
+// (src/llm/transformer.mm:822-840); at most num_nodes steps.
+__global__ void tree_mask_kernel(const int32_t* parents, uint32_t* mask, uint32_t num_nodes,
+                                 uint32_t words) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= num_nodes) return;
+    uint32_t* row = mask + size_t(i) * words;
+    for (uint32_t w = 0; w < words; w++) row[w] = 0;
+    row[i >> 5] |= 1u << (i & 31);
+    int32_t cur = parents[i];
+    for (uint32_t step = 0; step < num_nodes && cur >= 0 && cur < int32_t(num_nodes); step++) {
+        row[uint32_t(cur) >> 5] |= 1u << (uint32_t(cur) & 31);
+        cur = parents[cur];
+    }
+}
+
+}  // namespace
+
+int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes) {
+    if (!parents || !mask_words) return GRANITE_HIP_ENULL;
+    if (num_nodes == 0) return GRANITE_HIP_OK;
+    const uint32_t words = (num_nodes + 31) / 32;
+    tree_mask_kernel<<<dim3((num_nodes + 63) / 64), dim3(64), 0, ctx().stream>>>(
+        parents, mask_words, num_nodes, words);
+    return launch_status();
+}
+
+int launch_attention(const granite_hip_attention_args& a) {
+    if (!a.q || !a.out) return GRANITE_HIP_ENULL;
+    if (a.head_dim != kHeadDim) return GRANITE_HIP_EINVAL;
+    if (a.num_heads == 0 || a.num_kv_heads == 0 || a.num_heads % a.num_kv_heads != 0)
+        return GRANITE_HIP_EINVAL;
+    if ((a.q_dtype != GRANITE_HIP_F32 && a.q_dtype != GRANITE_HIP_F16) ||
+        (a.out_dtype != GRANITE_HIP_F32 && a.out_dtype != GRANITE_HIP_F16))
+        return GRANITE_HIP_EINVAL;
+    if (a.seq_q == 0) return GRANITE_HIP_OK;
+    if (a.cache_len + a.extra_len == 0) return GRANITE_HIP_EINVAL;
+    if (a.cache_len > 0 && (!a.k_cache || !a.v_cache)) return GRANITE_HIP_ENULL;
+    if (a.extra_len > 0 && (!a.k_extra || !a.v_extra)) return GRANITE_HIP_ENULL;
+    if (a.block_table && a.block_size == 0) return GRANITE_HIP_EINVAL;
+    if (!a.block_table && a.cache_len > 0 && a.max_seq < a.cache_len) return GRANITE_HIP_EINVAL;
+    const size_t qes = a.q_dtype == GRANITE_HIP_F32 ? 4 : 2, oes = a.out_dtype == GRANITE_HIP_F32 ? 4 : 2;
+    if ((a.q_tok_stride * qes) % 16 || (a.q_head_stride * qes) % 16 ||
+        (reinterpret_cast<uintptr_t>(a.q) & 15) || (a.out_tok_stride * oes) % 16 ||
+        (a.out_head_stride * oes) % 16 || (reinterpret_cast<uintptr_t>(a.out) & 15))
+        return GRANITE_HIP_EINVAL;
+
+    AttnParams p{};
+    p.q = a.q;
+    p.out = a.out;
+    p.lse = a.lse;
+    p.q_tok_stride = a.q_tok_stride;
+    p.q_head_stride = a.q_head_stride;
+    p.out_tok_stride = a.out_tok_stride;
+    p.out_head_stride = a.out_head_stride;
+    p.k = static_cast<const uint16_t*>(a.k_cache);
+    p.v = static_cast<const uint16_t*>(a.v_cache);
+    p.table = a.block_table;
+    p.block_size = a.block_table ? a.block_size : 1;
+    p.bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz(p.block_size) : -1;
+    if (a.block_table) {
+        p.a_tok_stride = int64_t(a.num_kv_heads) * kHeadDim;
+        p.a_head_stride = kHeadDim;
+    } else {
+        p.a_tok_stride = kHeadDim;
+        p.a_head_stride = int64_t(a.max_seq) * kHeadDim;
+    }
+    p.cache_len = a.cache_len;
+    p.k_extra = static_cast<const uint16_t*>(a.k_extra);
+    p.v_extra = static_cast<const uint16_t*>(a.v_extra);
+    p.extra_len = a.extra_len;
+    p.mask_mode = a.mask_mode;
+    p.start_pos = a.start_pos;
+    p.seq_q = a.seq_q;
+    p.num_heads = a.num_heads;
+    p.group = a.num_heads / a.num_kv_heads;
+    p.scale_log2 = a.scale * kLog2e;
+
+    if (a.mask_mode == GRANITE_HIP_MASK_CAUSAL) {
+        if (a.extra_len != 0) return GRANITE_HIP_EUNSUPPORTED;
+    } else if (a.mask_mode == GRANITE_HIP_MASK_TREE) {
+        if (!a.parents) return GRANITE_HIP_ENULL;
+        if (a.extra_len == 0 || a.seq_q != a.extra_len) return GRANITE_HIP_EINVAL;
+        p.mask_words = (a.extra_len + 31) / 32;
+        const size_t need = size_t(a.extra_len) * p.mask_words * sizeof(uint32_t);
+        int rc = ensure_workspace(need);
+        if (rc != GRANITE_HIP_OK) return rc;
+        uint32_t* mask = static_cast<uint32_t*>(ctx().workspace);
+        rc = launch_tree_mask(a.parents, mask, a.extra_len);
+        if (rc != GRANITE_HIP_OK) return rc;
+        p.tree_mask = mask;
+    } else if (a.mask_mode != GRANITE_HIP_MASK_NONE) {
+        return GRANITE_HIP_EINVAL;
+    }
+
+    const uint32_t q_tiles = (a.seq_q + kBM - 1) / kBM;
+    if (q_tiles > 0x7FFFFFFFu / 2 || a.num_heads > 65535u) return GRANITE_HIP_EINVAL;
+    dim3 grid(q_tiles, a.num_heads), block(kThreads);
+    hipStream_t st = ctx().stream;
+    const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
+    if (qf32 && of32)
+        attention_tiles_kernel<true, true><<<grid, block, 0, st>>>(p);
+    else if (qf32 && !of32)
+        attention_tiles_kernel<true, false><<<grid, block, 0, st>>>(p);
+    else if (!qf32 && of32)
+        attention_tiles_kernel<false, true><<<grid, block, 0, st>>>(p);
+    else
+        attention_tiles_kernel<false, false><<<grid, block, 0, st>>>(p);
+    return launch_status();
+}
+
+}  // namespace ghip

@@ -1,0 +1,234 @@
+"""Python mirror of the HipCompute class (the MetalCompute-shaped API of the
+HIP backend).  Method names, argument order and meaning follow
+include/granite/metal_compute.h:752-920 of the reference; every call goes
+straight to the C ABI in libgranite_hip.so.  Used by the tests and the
+benchmark; the C++ host layer in granite_amd/host is the same surface for C++
+callers.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import numpy as np
+
+from . import _capi
+from ._capi import (F16, F32, MASK_CAUSAL, MASK_NONE, MASK_TREE, MEM_DEVICE, ROUND_NEAREST,
+                    ROUND_TRUNCATE, AttentionArgs, DecodeArgs, check)
+
+
+class DeviceBuffer:
+    """A device allocation owned by the caller (Granite's MTL::Buffer stand-in)."""
+
+    def __init__(self, nbytes: int, kind: int = MEM_DEVICE):
+        self.nbytes = int(nbytes)
+        self.kind = kind
+        ptr = C.c_void_p()
+        check(_capi.load().granite_hip_malloc(C.byref(ptr), max(self.nbytes, 16), kind), "malloc")
+        self.ptr = ptr.value
+
+    @classmethod
+    def from_numpy(cls, arr: np.ndarray) -> "DeviceBuffer":
+        arr = np.ascontiguousarray(arr)
+        buf = cls(arr.nbytes)
+        buf.write(arr)
+        return buf
+
+    def write(self, arr: np.ndarray, offset: int = 0) -> None:
+        arr = np.ascontiguousarray(arr)
+        if offset + arr.nbytes > self.nbytes:
+            raise ValueError("write beyond the end of the buffer")
+        check(_capi.load().granite_hip_memcpy_h2d(self.ptr + offset, arr.ctypes.data, arr.nbytes),
+              "memcpy_h2d")
+
+    def read(self, dtype, shape, offset: int = 0) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        if offset + out.nbytes > self.nbytes:
+            raise ValueError("read beyond the end of the buffer")
+        check(_capi.load().granite_hip_memcpy_d2h(out.ctypes.data, self.ptr + offset, out.nbytes),
+              "memcpy_d2h")
+        return out
+
+    def fill(self, byte: int) -> None:
+        check(_capi.load().granite_hip_memset(self.ptr, byte, self.nbytes), "memset")
+
+    def free(self) -> None:
+        if self.ptr:
+            check(_capi.load().granite_hip_free(self.ptr, self.kind), "free")
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            if getattr(self, "ptr", None) and _capi.load().granite_hip_is_initialized():
+                _capi.load().granite_hip_free(self.ptr, self.kind)
+        except Exception:
+            pass
+
+
+def _p(buf) -> Optional[int]:
+    if buf is None:
+        return None
+    return buf.ptr if isinstance(buf, DeviceBuffer) else int(buf)
+
+
+class HipCompute:
+    """One in-order queue of attention / KV work on one MI355X."""
+
+    def __init__(self, device: int = 0):
+        self.lib = _capi.load()
+        self.device = device
+        self.initialize()
+
+    # ---- lifecycle (MetalCompute::initialize / shutdown / sync / commit)
+    def initialize(self) -> None:
+        check(self.lib.granite_hip_init(self.device), "init")
+
+    def shutdown(self) -> None:
+        check(self.lib.granite_hip_shutdown(), "shutdown")
+
+    def is_initialized(self) -> bool:
+        return bool(self.lib.granite_hip_is_initialized())
+
+    def sync(self) -> None:
+        check(self.lib.granite_hip_sync(), "sync")
+
+    def commit(self) -> None:
+        """Launches are submitted as they are made; nothing to flush."""
+
+    def device_info(self) -> _capi.DeviceInfo:
+        info = _capi.DeviceInfo()
+        check(self.lib.granite_hip_get_device_info(C.byref(info)), "get_device_info")
+        return info
+
+    def create_buffer(self, size: int, shared: bool = False) -> DeviceBuffer:
+        return DeviceBuffer(size, _capi.MEM_SHARED if shared else MEM_DEVICE)
+
+    # ---- timing
+    def event(self) -> int:
+        ev = C.c_void_p()
+        check(self.lib.granite_hip_event_create(C.byref(ev)), "event_create")
+        return ev.value
+
+    def record(self, ev: int) -> None:
+        check(self.lib.granite_hip_event_record(ev), "event_record")
+
+    def elapsed_ms(self, start: int, stop: int) -> float:
+        check(self.lib.granite_hip_event_synchronize(stop), "event_synchronize")
+        ms = C.c_float()
+        check(self.lib.granite_hip_event_elapsed_ms(start, stop, C.byref(ms)), "event_elapsed")
+        return ms.value
+
+    def destroy_event(self, ev: int) -> None:
+        check(self.lib.granite_hip_event_destroy(ev), "event_destroy")
+
+    # ---- KV cache
+    def kv_cache_append(self, cache_k, cache_v, new_k, new_v, num_kv_heads, head_dim,
+                        current_len, new_len, max_seq_len) -> None:
+        check(self.lib.granite_hip_kv_cache_append(_p(cache_k), _p(cache_v), _p(new_k), _p(new_v),
+                                                   num_kv_heads, head_dim, current_len, new_len,
+                                                   max_seq_len), "kv_cache_append")
+
+    def kv_cache_append_ex(self, cache_k, cache_v, new_k, new_v, src_dtype, src_tok_stride,
+                           src_head_stride, num_kv_heads, head_dim, current_len, new_len,
+                           max_seq_len, rounding=ROUND_TRUNCATE) -> None:
+        check(self.lib.granite_hip_kv_cache_append_ex(
+            _p(cache_k), _p(cache_v), _p(new_k), _p(new_v), src_dtype, src_tok_stride,
+            src_head_stride, num_kv_heads, head_dim, current_len, new_len, max_seq_len, rounding),
+            "kv_cache_append_ex")
+
+    def paged_kv_cache_append(self, new_k, new_v, k_cache, v_cache, block_table, num_kv_heads,
+                              head_dim, start_pos, new_len, block_size) -> None:
+        check(self.lib.granite_hip_paged_kv_cache_append(
+            _p(new_k), _p(new_v), _p(k_cache), _p(v_cache), _p(block_table), num_kv_heads,
+            head_dim, start_pos, new_len, block_size), "paged_kv_cache_append")
+
+    def paged_kv_cache_append_ex(self, new_k, new_v, src_dtype, src_tok_stride, src_head_stride,
+                                 k_cache, v_cache, block_table, num_kv_heads, head_dim, start_pos,
+                                 new_len, block_size, rounding=ROUND_TRUNCATE) -> None:
+        check(self.lib.granite_hip_paged_kv_cache_append_ex(
+            _p(new_k), _p(new_v), src_dtype, src_tok_stride, src_head_stride, _p(k_cache),
+            _p(v_cache), _p(block_table), num_kv_heads, head_dim, start_pos, new_len, block_size,
+            rounding), "paged_kv_cache_append_ex")
+
+    def paged_kv_gather(self, dst_k, dst_v, k_cache, v_cache, block_table, num_kv_heads, head_dim,
+                        length, block_size, max_seq_len) -> None:
+        check(self.lib.granite_hip_paged_kv_gather(
+            _p(dst_k), _p(dst_v), _p(k_cache), _p(v_cache), _p(block_table), num_kv_heads,
+            head_dim, length, block_size, max_seq_len), "paged_kv_gather")
+
+    # ---- attention (reference-shaped entry points)
+    def multihead_attention(self, Q, K, V, output, num_heads, num_kv_heads, seq_q, seq_kv,
+                            head_dim, scale, max_seq=0) -> None:
+        check(self.lib.granite_hip_multihead_attention(
+            _p(Q), _p(K), _p(V), _p(output), num_heads, num_kv_heads, seq_q, seq_kv, head_dim,
+            scale, max_seq), "multihead_attention")
+
+    def attention_tree(self, Q, K_cache, V_cache, K_tree, V_tree, parent_indices, output,
+                       num_heads, num_kv_heads, num_nodes, cache_len, head_dim, scale) -> None:
+        check(self.lib.granite_hip_attention_tree(
+            _p(Q), _p(K_cache), _p(V_cache), _p(K_tree), _p(V_tree), _p(parent_indices),
+            _p(output), num_heads, num_kv_heads, num_nodes, cache_len, head_dim, scale),
+            "attention_tree")
+
+    def paged_attention_decode(self, Q, K_cache, V_cache, block_table, output, num_heads,
+                               num_kv_heads, seq_len, head_dim, block_size, scale) -> None:
+        check(self.lib.granite_hip_paged_attention_decode(
+            _p(Q), _p(K_cache), _p(V_cache), _p(block_table), _p(output), num_heads, num_kv_heads,
+            seq_len, head_dim, block_size, scale), "paged_attention_decode")
+
+    def batched_paged_attention_decode(self, Q, K_cache, V_cache, block_tables, seq_lens, output,
+                                       batch_size, num_heads, num_kv_heads, head_dim, block_size,
+                                       max_blocks_per_seq, scale) -> None:
+        check(self.lib.granite_hip_batched_paged_attention_decode(
+            _p(Q), _p(K_cache), _p(V_cache), _p(block_tables), _p(seq_lens), _p(output),
+            batch_size, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq, scale),
+            "batched_paged_attention_decode")
+
+    # ---- attention (general forms)
+    def decode_attention(self, *, q, q_dtype, k_cache, v_cache, out, batch_size, num_heads,
+                         num_kv_heads, head_dim, scale, block_tables=None, seq_lens=None,
+                         lse=None, block_size=0, max_blocks_per_seq=0, max_seq=0,
+                         fixed_seq_len=0, chunk_tokens=0) -> None:
+        a = DecodeArgs(q=_p(q), q_dtype=q_dtype, k_cache=_p(k_cache), v_cache=_p(v_cache),
+                       block_tables=_p(block_tables), seq_lens=_p(seq_lens), out=_p(out),
+                       lse=_p(lse), batch_size=batch_size, num_heads=num_heads,
+                       num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size,
+                       max_blocks_per_seq=max_blocks_per_seq, max_seq=max_seq, scale=scale,
+                       fixed_seq_len=fixed_seq_len, chunk_tokens=chunk_tokens)
+        check(self.lib.granite_hip_decode_attention(C.byref(a)), "decode_attention")
+
+    def attention(self, *, q, q_dtype, q_tok_stride, q_head_stride, out, out_dtype,
+                  out_tok_stride, out_head_stride, seq_q, num_heads, num_kv_heads, head_dim, scale,
+                  k_cache=None, v_cache=None, cache_len=0, max_seq=0, block_table=None,
+                  block_size=0, k_extra=None, v_extra=None, extra_len=0, parents=None,
+                  mask_mode=MASK_CAUSAL, start_pos=0, lse=None) -> None:
+        a = AttentionArgs(q=_p(q), q_dtype=q_dtype, q_tok_stride=q_tok_stride,
+                          q_head_stride=q_head_stride, out=_p(out), out_dtype=out_dtype,
+                          out_tok_stride=out_tok_stride, out_head_stride=out_head_stride,
+                          lse=_p(lse), k_cache=_p(k_cache), v_cache=_p(v_cache),
+                          block_table=_p(block_table), block_size=block_size, max_seq=max_seq,
+                          cache_len=cache_len, k_extra=_p(k_extra), v_extra=_p(v_extra),
+                          extra_len=extra_len, parents=_p(parents), mask_mode=mask_mode,
+                          start_pos=start_pos, seq_q=seq_q, num_heads=num_heads,
+                          num_kv_heads=num_kv_heads, head_dim=head_dim, scale=scale)
+        check(self.lib.granite_hip_attention(C.byref(a)), "attention")
+
+    def build_tree_mask(self, parent_indices, mask_words, num_nodes) -> None:
+        check(self.lib.granite_hip_build_tree_mask(_p(parent_indices), _p(mask_words), num_nodes),
+              "build_tree_mask")
+
+
+_instance: Optional[HipCompute] = None
+
+
+def get_hip_compute(device: int = 0) -> HipCompute:
+    """Process-wide instance, created on first use (get_metal_compute() analogue,
+    src/backend/metal/metal_compute.mm:2721-2745)."""
+    global _instance
+    if _instance is None:
+        _instance = HipCompute(device)
+    return _instance
+
+
+__all__ = ["DeviceBuffer", "HipCompute", "get_hip_compute", "F16", "F32", "MASK_CAUSAL",
+           "MASK_NONE", "MASK_TREE", "ROUND_NEAREST", "ROUND_TRUNCATE"]

@@ -1,0 +1,294 @@
+/*
+ * granite_hip.h -- C ABI of the MI355X (gfx950) attention backend for Granite.
+ *
+ * One shared library, libgranite_hip.so, exports everything below.  The
+ * signatures use plain pointers and integers only, so the library can be
+ * bound from C++ (the HipCompute / HipBackend classes of the host layer),
+ * from ctypes, or from any other FFI.  Each entry point names the interface
+ * of the reference that it stands in for (paths relative to the reference
+ * tree).
+ *
+ * Conventions
+ *   - every function returns 0 on success, a GRANITE_HIP_E* code (negative)
+ *     for a rejected argument, or a positive hipError_t value;
+ *     granite_hip_error_string() renders either;
+ *   - all device pointers come from granite_hip_malloc() (or any other HIP
+ *     allocation on the same device);
+ *   - launches are enqueued on the library's single in-order stream and
+ *     return immediately; results are valid after granite_hip_sync(), exactly
+ *     like MetalCompute::sync() (src/backend/metal/metal_compute.mm:150-207);
+ *   - "half" means IEEE binary16 stored as uint16_t;
+ *   - head_dim must be 128 for the attention entry points (InvalidArgument
+ *     otherwise, mirroring metal_compute.mm:2556-2559); the KV append/gather
+ *     entry points accept any head_dim that is a multiple of 8.
+ *
+ * Layouts (D = head_dim, G = num_heads / num_kv_heads)
+ *   contiguous cache   [num_kv_heads, max_seq, D] half   (src/llm/kv_cache.cpp:20-25)
+ *   paged pool         [num_blocks*block_size, num_kv_heads, D] half
+ *                      (src/llm/paged_kv_cache.cpp:44-49); logical token p of a
+ *                      sequence lives in row block_table[p / bs] * bs + p % bs
+ */
+#ifndef GRANITE_HIP_H
+#define GRANITE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes ------------------------------------------------------- */
+#define GRANITE_HIP_OK 0
+#define GRANITE_HIP_EINVAL (-1)      /* ErrorCode::InvalidArgument */
+#define GRANITE_HIP_ENOTINIT (-2)    /* ErrorCode::BackendNotInitialized */
+#define GRANITE_HIP_ENOMEM (-3)      /* ErrorCode::AllocationFailed */
+#define GRANITE_HIP_EUNSUPPORTED (-4)/* ErrorCode::NotImplemented */
+#define GRANITE_HIP_ENULL (-5)       /* ErrorCode::NullPointer */
+#define GRANITE_HIP_EOVERFLOW (-6)   /* KV cache overflow (kv_cache.cpp:61-65) */
+
+/* element types of Q / output tensors */
+#define GRANITE_HIP_F32 0
+#define GRANITE_HIP_F16 1
+
+/* float -> half conversion used by the append entry points */
+#define GRANITE_HIP_ROUND_TRUNCATE 0 /* Granite's CPU fp32_to_fp16 (src/llm/math_ops.cpp:45-54) */
+#define GRANITE_HIP_ROUND_NEAREST 1  /* Granite's GPU kernels, half(x) (metal_shaders_attention.h:124) */
+
+/* memory kinds, same order as granite::MemoryType (include/granite/types.h:131-135) */
+#define GRANITE_HIP_MEM_DEVICE 0
+#define GRANITE_HIP_MEM_SHARED 1  /* pinned host memory, device-visible */
+#define GRANITE_HIP_MEM_MANAGED 2 /* device memory + host mirror handled by the C++ backend */
+
+/* mask modes of granite_hip_attention() */
+#define GRANITE_HIP_MASK_NONE 0   /* every key visible */
+#define GRANITE_HIP_MASK_CAUSAL 1 /* key k visible iff k <= start_pos + q */
+#define GRANITE_HIP_MASK_TREE 2   /* cache keys visible; extra keys by ancestor walk */
+
+/* ---- backend: lifecycle, memory, stream ------------------------------- *
+ * Stand in for the parts of IComputeBackend that touch the device
+ * (include/granite/backend.h:30-183: initialize/shutdown, create_buffer,
+ * write_buffer/read_buffer/copy_buffer, wait_for_completion) and for
+ * MetalCompute::{initialize,shutdown,sync,commit,create_buffer}
+ * (include/granite/metal_compute.h:29-43, 944). */
+typedef struct granite_hip_device_info {
+    char name[128];
+    char arch[32];
+    size_t total_memory;
+    size_t max_buffer_size;
+    size_t shared_memory_per_block;
+    int max_threads_per_block;
+    int wavefront_size;
+    int compute_units;
+    int clock_khz;
+} granite_hip_device_info;
+
+int granite_hip_init(int device);
+int granite_hip_shutdown(void);
+int granite_hip_is_initialized(void);
+int granite_hip_get_device_info(granite_hip_device_info *info);
+const char *granite_hip_error_string(int code);
+const char *granite_hip_version(void);
+
+int granite_hip_malloc(void **ptr, size_t bytes, int memory_kind);
+int granite_hip_free(void *ptr, int memory_kind);
+int granite_hip_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int granite_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int granite_hip_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int granite_hip_memset(void *dst, int value, size_t bytes);
+int granite_hip_sync(void);
+/* Use `stream` (a hipStream_t) for all later launches; NULL restores the
+ * library's own stream. */
+int granite_hip_set_stream(void *stream);
+void *granite_hip_get_stream(void);
+
+/* Timing on the launch stream (MetalCompute::enable_kernel_timing analogue,
+ * metal_compute.h:51-59): events are created, recorded on the launch stream
+ * and compared in milliseconds. */
+int granite_hip_event_create(void **event);
+int granite_hip_event_destroy(void *event);
+int granite_hip_event_record(void *event);
+int granite_hip_event_synchronize(void *event);
+int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ---- KV cache append / gather ----------------------------------------- */
+
+/* MetalCompute::kv_cache_append (include/granite/metal_compute.h:784-797;
+ * kernel metal_shaders_attention.h:102-125).  new_k/new_v: [new_len,
+ * num_kv_heads, D] float; cache_k/cache_v: contiguous cache.  Rows
+ * current_len .. current_len+new_len-1 are written; conversion is
+ * GRANITE_HIP_ROUND_TRUNCATE (the CPU path's, transformer.mm:1687-1688).
+ * current_len + new_len > max_seq_len -> GRANITE_HIP_EOVERFLOW. */
+int granite_hip_kv_cache_append(void *cache_k, void *cache_v, const void *new_k,
+                                const void *new_v, uint32_t num_kv_heads, uint32_t head_dim,
+                                uint32_t current_len, uint32_t new_len, uint32_t max_seq_len);
+
+/* General form.  src_dtype F32 (converted with `rounding`) or F16 (bit copy).
+ * Source element (token s, head h, d) is at s*src_tok_stride +
+ * h*src_head_stride + d, so [new_len,Hkv,D] (tok stride Hkv*D, head stride D)
+ * and KVCache::append's [Hkv,new_len,D] (src/llm/kv_cache.cpp:86-94; tok
+ * stride D, head stride new_len*D) are both covered. */
+int granite_hip_kv_cache_append_ex(void *cache_k, void *cache_v, const void *new_k,
+                                   const void *new_v, int src_dtype, int64_t src_tok_stride,
+                                   int64_t src_head_stride, uint32_t num_kv_heads,
+                                   uint32_t head_dim, uint32_t current_len, uint32_t new_len,
+                                   uint32_t max_seq_len, int rounding);
+
+/* MetalCompute::paged_kv_cache_append (metal_compute.h:887-898; kernel
+ * metal_shaders_attention.h:2142-2176).  new_k/new_v: [num_kv_heads, new_len,
+ * D] float; pools paged; block_table: int32[>= ceil((start_pos+new_len)/bs)].
+ * Conversion GRANITE_HIP_ROUND_TRUNCATE. */
+int granite_hip_paged_kv_cache_append(const void *new_k, const void *new_v, void *k_cache,
+                                      void *v_cache, const int32_t *block_table,
+                                      uint32_t num_kv_heads, uint32_t head_dim,
+                                      uint32_t start_pos, uint32_t new_len, uint32_t block_size);
+
+/* General form (strided source, F32 or F16 source, rounding choice). */
+int granite_hip_paged_kv_cache_append_ex(const void *new_k, const void *new_v, int src_dtype,
+                                         int64_t src_tok_stride, int64_t src_head_stride,
+                                         void *k_cache, void *v_cache,
+                                         const int32_t *block_table, uint32_t num_kv_heads,
+                                         uint32_t head_dim, uint32_t start_pos,
+                                         uint32_t new_len, uint32_t block_size, int rounding);
+
+/* Gather of logical tokens [0, len) of one sequence out of the paged pools
+ * into contiguous caches [num_kv_heads, max_seq_len, D] half (bit copy).  The
+ * device form of the per-call gather in src/llm/transformer.mm:1750-1763 and
+ * of sync_cpu_to_gpu_kv_cache (transformer.mm:4539-4620). */
+int granite_hip_paged_kv_gather(void *dst_k, void *dst_v, const void *k_cache,
+                                const void *v_cache, const int32_t *block_table,
+                                uint32_t num_kv_heads, uint32_t head_dim, uint32_t len,
+                                uint32_t block_size, uint32_t max_seq_len);
+
+/* ---- attention --------------------------------------------------------- */
+
+/* MetalCompute::multihead_attention (metal_compute.h:799-816;
+ * metal_compute.mm:2253-2378).  K, V: contiguous cache with row stride
+ * max_seq (0 = seq_kv).  seq_q == 1: decode, Q/out [num_heads, D] float.
+ * seq_q > 1: causal prefill with start_pos 0, Q/out [seq_q, num_heads, D]
+ * float (the layout the reference kernel indexes,
+ * metal_shaders_attention.h:1640-1660).  Semantics are the CPU path's
+ * (transformer.mm:1779-1840): no epsilon in the denominator, fp32 softmax. */
+int granite_hip_multihead_attention(const void *q, const void *k, const void *v, void *out,
+                                    uint32_t num_heads, uint32_t num_kv_heads, uint32_t seq_q,
+                                    uint32_t seq_kv, uint32_t head_dim, float scale,
+                                    uint32_t max_seq);
+
+/* MetalCompute::attention_tree (metal_compute.h:830-844; metal_compute.mm:2463-2529).
+ * Q/out [num_heads, num_nodes, D] float; k_cache/v_cache contiguous with row
+ * stride cache_len (as the reference kernel indexes them,
+ * metal_shaders_attention.h:1708-1709); k_tree/v_tree [num_kv_heads,
+ * num_nodes, D] half; parent_indices int32[num_nodes], -1 = root.  Node i sees
+ * the whole cache, itself and its ancestors (transformer.mm:822-840). */
+int granite_hip_attention_tree(const void *q, const void *k_cache, const void *v_cache,
+                               const void *k_tree, const void *v_tree,
+                               const int32_t *parent_indices, void *out, uint32_t num_heads,
+                               uint32_t num_kv_heads, uint32_t num_nodes, uint32_t cache_len,
+                               uint32_t head_dim, float scale);
+
+/* MetalCompute::paged_attention_decode (metal_compute.h:869-881;
+ * metal_compute.mm:2535-2621).  Q/out [num_heads, D] float. */
+int granite_hip_paged_attention_decode(const void *q, const void *k_cache, const void *v_cache,
+                                       const int32_t *block_table, void *out,
+                                       uint32_t num_heads, uint32_t num_kv_heads,
+                                       uint32_t seq_len, uint32_t head_dim,
+                                       uint32_t block_size, float scale);
+
+/* MetalCompute::batched_paged_attention_decode (metal_compute.h:906-920;
+ * metal_compute.mm:2658-2696).  Q/out [batch, num_heads, D] float;
+ * block_tables int32[batch, max_blocks_per_seq]; seq_lens int32[batch] (device
+ * memory); a sequence of length 0 leaves its output rows untouched. */
+int granite_hip_batched_paged_attention_decode(const void *q, const void *k_cache,
+                                               const void *v_cache,
+                                               const int32_t *block_tables,
+                                               const int32_t *seq_lens, void *out,
+                                               uint32_t batch_size, uint32_t num_heads,
+                                               uint32_t num_kv_heads, uint32_t head_dim,
+                                               uint32_t block_size,
+                                               uint32_t max_blocks_per_seq, float scale);
+
+/* Decode, general form: adds half-precision Q, a log-sum-exp output and a
+ * contiguous-cache variant to the two entry points above.
+ *   q            [batch, num_heads, D], q_dtype F32 or F16
+ *   out          [batch, num_heads, D] float
+ *   lse          float[batch, num_heads] or NULL; natural-log-sum-exp of the
+ *                scaled scores (no reference counterpart: the reference keeps
+ *                max and sum internal, metal_shaders_attention.h:3046-3048)
+ *   block_tables NULL selects the contiguous cache layout with row stride
+ *                max_seq (batch must be 1); otherwise paged
+ *   seq_lens     device int32[batch], bounded by max_blocks_per_seq*block_size
+ *                (paged) or max_seq (contiguous), from which the grid is
+ *                sized; NULL means every sequence has the host-known length
+ *                fixed_seq_len. */
+typedef struct granite_hip_decode_args {
+    const void *q;
+    int q_dtype;
+    const void *k_cache;
+    const void *v_cache;
+    const int32_t *block_tables;
+    const int32_t *seq_lens;
+    void *out;
+    float *lse;
+    uint32_t batch_size, num_heads, num_kv_heads, head_dim;
+    uint32_t block_size, max_blocks_per_seq; /* paged */
+    uint32_t max_seq;                        /* contiguous: row stride and length bound */
+    float scale;
+    uint32_t fixed_seq_len; /* used when seq_lens is NULL */
+    uint32_t chunk_tokens;  /* split-K chunk, multiple of 32; 0 = library default */
+} granite_hip_decode_args;
+
+int granite_hip_decode_attention(const granite_hip_decode_args *args);
+
+/* Prefill / chunked prefill / tree attention, general form.  One sequence.
+ * Keys are the concatenation of
+ *   segment A: `cache_len` tokens from the KV cache -- contiguous (block_table
+ *              NULL, row stride max_seq) or paged (block_table given);
+ *   segment B: `extra_len` tokens from k_extra/v_extra [num_kv_heads,
+ *              extra_len, D] half (tree nodes; NULL/0 when unused).
+ * mask_mode CAUSAL: key k (index in the concatenation) visible iff
+ *              k <= start_pos + q                       (transformer.mm:1797-1806)
+ * mask_mode TREE:  segment A fully visible, key j of segment B visible to
+ *              query i iff j == i or j is an ancestor of i via parents[]
+ *              (transformer.mm:2066-2090, 822-840); seq_q must equal extra_len.
+ * Q element (token t, head h, d) at t*q_tok_stride + h*q_head_stride + d;
+ * same for out with its strides; lse float[num_heads, seq_q] or NULL. */
+typedef struct granite_hip_attention_args {
+    const void *q;
+    int q_dtype;
+    int64_t q_tok_stride, q_head_stride;
+    void *out;
+    int out_dtype;
+    int64_t out_tok_stride, out_head_stride;
+    float *lse;
+    const void *k_cache;
+    const void *v_cache;
+    const int32_t *block_table;
+    uint32_t block_size;
+    uint32_t max_seq;
+    uint32_t cache_len;
+    const void *k_extra;
+    const void *v_extra;
+    uint32_t extra_len;
+    const int32_t *parents;
+    int mask_mode;
+    uint32_t start_pos;
+    uint32_t seq_q, num_heads, num_kv_heads, head_dim;
+    float scale;
+} granite_hip_attention_args;
+
+int granite_hip_attention(const granite_hip_attention_args *args);
+
+/* Ancestor bit mask from parent pointers (transformer.mm:822-840): row i holds
+ * ceil(num_nodes/32) uint32 words, bit j of row i set iff node i may attend
+ * node j.  The walk stops after num_nodes steps, so a malformed parent array
+ * cannot hang the device. */
+int granite_hip_build_tree_mask(const int32_t *parent_indices, uint32_t *mask_words,
+                                uint32_t num_nodes);
+
+/* Bytes of device scratch the library keeps for split-K partial results. */
+size_t granite_hip_workspace_bytes(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GRANITE_HIP_H */
