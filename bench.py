@@ -1,0 +1,398 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Prints ONE JSON line.  The headline (`metric`/`value`) is paged-KV batched
+decode attention (64 sequences, context U[256, 8192], 32 query heads, 8 KV
+heads, D=128, block 16) in GB/s of algorithmic traffic; the prefill-side
+figures (TFLOP/s of the causal prefill and of the chunked prefill over a
+paged cache) and the two latency-bound workloads ride along under
+`workloads`.  A "step" is one pass of the hot path over one batch of
+synthetic input that is already resident in HBM.
+
+Every workload carries
+  roofline      for its dominant kernel: algorithmic bytes (or flops) per
+                launch / the kernel's mean duration, measured with HIP events
+                on the launch stream (the library's per-kernel timer);
+  cpu_baseline  the CPU restatement of Granite's CPU attention (the oracle)
+                timed on this host on a bounded sample, with the thread count.
+The oracle is only the checker and the baseline here; the measured path is
+the HIP library.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT, ROOT / "tests"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file (see profiles/); None until measured.
+MEASURED_TRAFFIC = {
+    "paged_decode": None,
+    "prefill": None,
+    "chunked_prefill": None,
+}
+
+
+def log(msg: str) -> None:
+    print(msg, file=sys.stderr, flush=True)
+
+
+class Timer:
+    """Times K back-to-back steps with events on the launch stream."""
+
+    def __init__(self, gpu):
+        self.gpu = gpu
+
+    def run(self, step, warmup: int, steps: int):
+        gpu = self.gpu
+        for _ in range(warmup):
+            step()
+        gpu.sync()
+        # whole-job time: K steps back to back
+        e0, e1 = gpu.event(), gpu.event()
+        t0 = time.perf_counter()
+        gpu.record(e0)
+        for _ in range(steps):
+            step()
+        gpu.record(e1)
+        gpu.sync()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        ev_ms = gpu.elapsed_ms(e0, e1)
+        gpu.destroy_event(e0)
+        gpu.destroy_event(e1)
+        # per-kernel durations: same K steps with the library's kernel timer on
+        gpu.reset_kernel_timing()
+        gpu.enable_kernel_timing(True)
+        for _ in range(steps):
+            step()
+        gpu.sync()
+        stats = gpu.get_kernel_timing_stats()
+        gpu.enable_kernel_timing(False)
+        return ev_ms / steps, wall_ms / steps, {k: (ms / max(n, 1), n) for k, (ms, n) in stats.items()}
+
+
+def roofline(bound: str, work: float, kernel_ms: float, traffic):
+    if bound == "hbm":
+        achieved = work / (kernel_ms * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic}
+    achieved = work / (kernel_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic}
+
+
+def max_err(got, want):
+    d = np.abs(np.asarray(got, np.float64) - np.asarray(want, np.float64))
+    return float(d.max(initial=0.0))
+
+
+# ---------------------------------------------------------------------------
+# workloads
+# ---------------------------------------------------------------------------
+
+def bench_paged_decode(gpu, steps, warmup, cpu):
+    from granite_amd import F16, DeviceBuffer, workloads as W
+    dev = DeviceBuffer.from_numpy
+    t0 = time.perf_counter()
+    c = W.make_paged_decode()
+    log(f"[paged_decode] inputs: {int(c.seq_lens.sum())} tokens, pool {c.k_pool.nbytes * 2 / 2**30:.2f} GiB "
+        f"({time.perf_counter() - t0:.1f}s)")
+    B, hq = c.batch, c.num_heads
+    bufs = dict(q=dev(c.q), k=dev(c.k_pool), v=dev(c.v_pool), t=dev(c.block_tables), l=dev(c.seq_lens))
+    out, lse = dev(np.zeros((B, hq, 128), np.float32)), dev(np.zeros((B, hq), np.float32))
+
+    def step():
+        gpu.decode_attention(q=bufs["q"], q_dtype=F16, k_cache=bufs["k"], v_cache=bufs["v"],
+                             block_tables=bufs["t"], seq_lens=bufs["l"], out=out, lse=lse, batch_size=B,
+                             num_heads=hq, num_kv_heads=c.num_kv_heads, head_dim=128, scale=c.scale,
+                             block_size=c.block_size, max_blocks_per_seq=c.max_blocks)
+
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    nbytes = c.algorithmic_bytes()
+    res = {
+        "workload": "paged_decode_b64_ctx256-8192_hq32_hkv8_d128_bs16",
+        "metric": "paged_decode_attn_GBps", "unit": "GB/s", "value": round(nbytes / (ms * 1e-3) / 1e9, 1),
+        "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
+        "algorithmic_bytes": nbytes, "flops": c.flops(), "dtype": "f16 K/V, f32 accumulate",
+        "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+        "roofline": roofline("hbm", nbytes, kern["decode_splitk"][0], MEASURED_TRAFFIC["paged_decode"]),
+    }
+    res["roofline"]["kernel"] = "decode_splitk_kernel"
+    if cpu:
+        import oracle_bind
+        oracle = oracle_bind.load()
+        q32 = c.q.astype(np.float32)
+        t0 = time.perf_counter()
+        want, want_lse = oracle.batched_paged_decode(q32, c.k_pool, c.v_pool, c.block_tables, c.seq_lens,
+                                                     c.block_size, c.scale)
+        cpu_s = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": round(nbytes / cpu_s / 1e9, 3), "unit": "GB/s",
+                               "cores": oracle.lib.go_get_num_threads(), "kind": "port",
+                               "seconds": round(cpu_s, 2),
+                               "sample": "the whole workload (all 64 sequences), one pass"}
+        res["parity"] = {"max_abs_err": max_err(out.read(np.float32, (B, hq, 128)), want),
+                         "max_lse_err": max_err(lse.read(np.float32, (B, hq)), want_lse)}
+    return res
+
+
+def bench_prefill(gpu, steps, warmup, cpu):
+    from granite_amd import F16, MASK_CAUSAL, DeviceBuffer, workloads as W
+    dev = DeviceBuffer.from_numpy
+    c = W.make_prefill()
+    S, hq, hkv = c.seq, c.num_heads, c.num_kv_heads
+    dq, dk, dv = dev(c.q), dev(c.k_cache), dev(c.v_cache)
+    out, lse = dev(np.zeros((S, hq, 128), np.float16)), dev(np.zeros((hq, S), np.float32))
+
+    def step():
+        gpu.attention(q=dq, q_dtype=F16, q_tok_stride=hq * 128, q_head_stride=128, out=out, out_dtype=F16,
+                      out_tok_stride=hq * 128, out_head_stride=128, lse=lse, seq_q=S, num_heads=hq,
+                      num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=dk, v_cache=dv, cache_len=S,
+                      max_seq=c.max_seq, mask_mode=MASK_CAUSAL, start_pos=0)
+
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    flops = c.flops()
+    res = {
+        "workload": "causal_prefill_s2048_hq32_hkv8_d128", "metric": "prefill_attn_TFLOPs", "unit": "TFLOP/s",
+        "value": round(flops / (ms * 1e-3) / 1e12, 2), "ms_per_step": round(ms, 4),
+        "wall_ms_per_step": round(wall_ms, 4), "flops": flops, "algorithmic_bytes": c.algorithmic_bytes(),
+        "dtype": "f16 MFMA, f32 accumulate", "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+        "roofline": roofline("mfma", flops, kern["attention_tiles"][0], MEASURED_TRAFFIC["prefill"]),
+    }
+    res["roofline"]["kernel"] = "attention_tiles_kernel"
+    if cpu:
+        import oracle_bind
+        oracle = oracle_bind.load()
+        rows = list(range(0, S, 16))  # every 16th query row, all heads
+        k = np.ascontiguousarray(np.transpose(c.k_cache, (1, 0, 2))).astype(np.float32)
+        v = np.ascontiguousarray(np.transpose(c.v_cache, (1, 0, 2))).astype(np.float32)
+        got = out.read(np.float16, (S, hq, 128)).astype(np.float32)
+        got_lse = lse.read(np.float32, (hq, S))
+        t0 = time.perf_counter()
+        err = lerr = 0.0
+        sample_flops = 0
+        for r in rows:
+            want, wl = oracle.attention_core(c.q[None, r:r + 1].astype(np.float32), k[:r + 1], v[:r + 1], r,
+                                             c.scale)
+            sample_flops += 4 * hq * 128 * (r + 1)
+            err = max(err, max_err(got[r], want[0, 0]))
+            lerr = max(lerr, max_err(got_lse[:, r], wl[0, :, 0]))
+        cpu_s = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": round(sample_flops / cpu_s / 1e12, 5), "unit": "TFLOP/s",
+                               "cores": oracle.lib.go_get_num_threads(), "kind": "port",
+                               "seconds": round(cpu_s, 2),
+                               "sample": f"every 16th query row ({len(rows)} rows x {hq} heads), "
+                                         "attention core only (no cache gather)"}
+        res["parity"] = {"max_abs_err": err, "max_lse_err": lerr}
+    return res
+
+
+def bench_chunked_prefill(gpu, steps, warmup, cpu):
+    from granite_amd import F16, MASK_CAUSAL, DeviceBuffer, workloads as W
+    import ref64
+    dev = DeviceBuffer.from_numpy
+    c = W.make_chunked_prefill()
+    hq, hkv, bs, prefix, chunk = c.num_heads, c.num_kv_heads, c.block_size, c.prefix_len, c.chunk
+    total = prefix + chunk
+    dq, dk, dv, dt = dev(c.q), dev(c.k_pool), dev(c.v_pool), dev(c.block_table)
+    dkn, dvn = dev(c.k_new), dev(c.v_new)
+    out, lse = dev(np.zeros((chunk, hq, 128), np.float16)), dev(np.zeros((hq, chunk), np.float32))
+
+    def step():  # append the chunk's K/V into its fresh blocks, then attend
+        gpu.paged_kv_cache_append_ex(dkn, dvn, F16, hkv * 128, 128, dk, dv, dt, hkv, 128, prefix, chunk, bs)
+        gpu.attention(q=dq, q_dtype=F16, q_tok_stride=hq * 128, q_head_stride=128, out=out, out_dtype=F16,
+                      out_tok_stride=hq * 128, out_head_stride=128, lse=lse, seq_q=chunk, num_heads=hq,
+                      num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=dk, v_cache=dv, cache_len=total,
+                      block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
+
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    flops = c.flops()
+    res = {
+        "workload": "chunked_prefill_prefix32768_chunk512_hq64_hkv8_d128_bs32",
+        "metric": "prefill_attn_TFLOPs", "unit": "TFLOP/s", "value": round(flops / (ms * 1e-3) / 1e12, 2),
+        "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4), "flops": flops,
+        "algorithmic_bytes": c.algorithmic_bytes(), "dtype": "f16 MFMA, f32 accumulate",
+        "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+        "roofline": roofline("mfma", flops, kern["attention_tiles"][0], MEASURED_TRAFFIC["chunked_prefill"]),
+    }
+    res["roofline"]["kernel"] = "attention_tiles_kernel"
+    if cpu:
+        import oracle_bind
+        oracle = oracle_bind.load()
+        k_all = ref64.gather_paged(c.k_pool, c.block_table, bs, total).copy()
+        v_all = ref64.gather_paged(c.v_pool, c.block_table, bs, total).copy()
+        k_all[prefix:], v_all[prefix:] = c.k_new, c.v_new
+        k32, v32 = k_all.astype(np.float32), v_all.astype(np.float32)
+        got = out.read(np.float16, (chunk, hq, 128)).astype(np.float32)
+        got_lse = lse.read(np.float32, (hq, chunk))
+        rows = [0, 73, 146, 219, 292, 365, 438, 511]
+        t0 = time.perf_counter()
+        err = lerr = 0.0
+        sample_flops = 0
+        for r in rows:
+            want, wl = oracle.attention_core(c.q[None, r:r + 1].astype(np.float32), k32[:prefix + r + 1],
+                                             v32[:prefix + r + 1], prefix + r, c.scale)
+            sample_flops += 4 * hq * 128 * (prefix + r + 1)
+            err = max(err, max_err(got[r], want[0, 0]))
+            lerr = max(lerr, max_err(got_lse[:, r], wl[0, :, 0]))
+        cpu_s = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": round(sample_flops / cpu_s / 1e12, 5), "unit": "TFLOP/s",
+                               "cores": oracle.lib.go_get_num_threads(), "kind": "port",
+                               "seconds": round(cpu_s, 2),
+                               "sample": f"{len(rows)} of 512 query rows x {hq} heads, attention core only"}
+        res["parity"] = {"max_abs_err": err, "max_lse_err": lerr}
+    return res
+
+
+def bench_tree(gpu, steps, warmup, cpu):
+    from granite_amd import F32, MASK_TREE, DeviceBuffer, workloads as W
+    dev = DeviceBuffer.from_numpy
+    c = W.make_tree()
+    hq, hkv, n = c.num_heads, c.num_kv_heads, c.num_nodes
+    b = dict(q=dev(c.q), k=dev(c.k_pool), v=dev(c.v_pool), t=dev(c.block_table), kt=dev(c.k_tree),
+             vt=dev(c.v_tree), p=dev(c.parents))
+    out, lse = dev(np.zeros((hq, n, 128), np.float32)), dev(np.zeros((hq, n), np.float32))
+
+    def step():
+        gpu.attention(q=b["q"], q_dtype=F32, q_tok_stride=128, q_head_stride=n * 128, out=out, out_dtype=F32,
+                      out_tok_stride=128, out_head_stride=n * 128, lse=lse, seq_q=n, num_heads=hq,
+                      num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=b["k"], v_cache=b["v"],
+                      cache_len=c.prefix_len, block_table=b["t"], block_size=c.block_size, k_extra=b["kt"],
+                      v_extra=b["vt"], extra_len=n, parents=b["p"], mask_mode=MASK_TREE)
+
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    res = {
+        "workload": "tree_prefix4096_nodes64_hq32_hkv8_d128_bs16", "metric": "tree_attn_latency_us", "unit": "us",
+        "value": round(ms * 1e3, 2), "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
+        "flops": c.flops(), "algorithmic_bytes": c.algorithmic_bytes(),
+        "GBps": round(c.algorithmic_bytes() / (ms * 1e-3) / 1e9, 1),
+        "TFLOPs": round(c.flops() / (ms * 1e-3) / 1e12, 2),
+        "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+        "note": "launch/latency bound (19 MB, 4.3 GFLOP); reported, no roofline target",
+    }
+    if cpu:
+        import oracle_bind
+        oracle = oracle_bind.load()
+        q = np.transpose(c.q, (1, 0, 2))[None]
+        kt = np.transpose(c.k_tree, (1, 0, 2))[None].astype(np.float32)
+        vt = np.transpose(c.v_tree, (1, 0, 2))[None].astype(np.float32)
+        t0 = time.perf_counter()
+        ctx, wl = oracle.attention_tree(q, c.k_pool, c.v_pool, kt, vt, c.parents, c.prefix_len, c.scale,
+                                        table=c.block_table, block_size=c.block_size)
+        cpu_s = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": round(cpu_s * 1e6, 1), "unit": "us",
+                               "cores": oracle.lib.go_get_num_threads(), "kind": "port",
+                               "sample": "the whole workload, one pass (incl. the prefix gather)"}
+        res["parity"] = {"max_abs_err": max_err(out.read(np.float32, (hq, n, 128)), np.transpose(ctx[0], (1, 0, 2))),
+                         "max_lse_err": max_err(lse.read(np.float32, (hq, n)), wl[0])}
+    return res
+
+
+def bench_decode_contiguous(gpu, steps, warmup, cpu):
+    from granite_amd import F32, DeviceBuffer, workloads as W
+    dev = DeviceBuffer.from_numpy
+    c = W.make_decode_contiguous()
+    dq, dk, dv = dev(c.q), dev(c.k_cache), dev(c.v_cache)
+    out, lse = dev(np.zeros((32, 128), np.float32)), dev(np.zeros(32, np.float32))
+
+    def step():
+        gpu.decode_attention(q=dq, q_dtype=F32, k_cache=dk, v_cache=dv, out=out, lse=lse, batch_size=1,
+                             num_heads=32, num_kv_heads=8, head_dim=128, scale=c.scale, max_seq=c.max_seq,
+                             fixed_seq_len=c.seq_kv)
+
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    res = {
+        "workload": "decode_contiguous_ctx512_hq32_hkv8_d128", "metric": "decode_attn_latency_us", "unit": "us",
+        "value": round(ms * 1e3, 2), "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
+        "algorithmic_bytes": c.algorithmic_bytes(), "GBps": round(c.algorithmic_bytes() / (ms * 1e-3) / 1e9, 1),
+        "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+        "note": "2 MB of traffic: launch-latency bound and cache resident; reported, no roofline target",
+    }
+    if cpu:
+        import oracle_bind
+        oracle = oracle_bind.load()
+        reps = 20
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            want, wl = oracle.attention_cached(c.q[None, None], c.k_cache, c.v_cache, c.seq_kv, c.seq_kv - 1,
+                                               c.scale)
+        cpu_s = (time.perf_counter() - t0) / reps
+        res["cpu_baseline"] = {"value": round(cpu_s * 1e6, 1), "unit": "us",
+                               "cores": oracle.lib.go_get_num_threads(), "kind": "port",
+                               "sample": f"the whole workload, mean of {reps} passes (incl. the cache gather)"}
+        res["parity"] = {"max_abs_err": max_err(out.read(np.float32, (32, 128)), want[0, 0]),
+                         "max_lse_err": max_err(lse.read(np.float32, (32,)), wl[0, :, 0])}
+    return res
+
+
+WORKLOADS = {
+    "paged_decode": bench_paged_decode,
+    "prefill": bench_prefill,
+    "chunked_prefill": bench_chunked_prefill,
+    "tree": bench_tree,
+    "decode_contiguous": bench_decode_contiguous,
+}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on exactly one GPU (--gpus 1); the attention path has no "
+              "cross-GPU step (it would shard by KV head or by sequence).", file=sys.stderr)
+        return 2
+
+    from granite_amd import get_hip_compute
+    gpu = get_hip_compute(0)
+    info = gpu.device_info()
+    log(f"device: {info.name.decode()} {info.arch.decode()} CUs={info.compute_units} clock={info.clock_khz} kHz")
+
+    names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+    results = {}
+    for name in names:
+        t0 = time.perf_counter()
+        results[name] = WORKLOADS[name](gpu, args.steps, args.warmup, not args.no_cpu)
+        log(f"[{name}] {results[name]['value']} {results[name]['unit']} "
+            f"({results[name]['ms_per_step']} ms/step; {time.perf_counter() - t0:.1f}s total)")
+
+    head = results.get("paged_decode") or results[names[0]]
+    line = {
+        "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": head["unit"] != "us", "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": head["workload"], "device": info.name.decode(), "arch": info.arch.decode(),
+                   "compute_units": info.compute_units},
+    }
+    if "roofline" in head:
+        line["roofline"] = head["roofline"]
+    if "cpu_baseline" in head:
+        line["cpu_baseline"] = head["cpu_baseline"]
+    if "parity" in head:
+        line["parity"] = head["parity"]
+    line["workloads"] = results
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -118,6 +118,10 @@ SIGNATURES = {
     "granite_hip_event_record": (_int, [_vp]),
     "granite_hip_event_synchronize": (_int, [_vp]),
     "granite_hip_event_elapsed_ms": (_int, [_vp, _vp, C.POINTER(_f32)]),
+    "granite_hip_enable_kernel_timing": (_int, [_int]),
+    "granite_hip_reset_kernel_timing": (_int, []),
+    "granite_hip_get_kernel_timing": (_int, [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
+    "granite_hip_kernel_timing_names": (_int, [C.c_char_p, C.c_size_t]),
     "granite_hip_kv_cache_append": (_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "granite_hip_kv_cache_append_ex": (
         _int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _u32, _u32, _u32, _u32, _u32, _int]),

@@ -5,6 +5,9 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <string>
+#include <vector>
 
 #include "common.h"
 
@@ -32,6 +35,68 @@ int ensure_workspace(size_t bytes) {
     }
     c.workspace_bytes = want;
     return GRANITE_HIP_OK;
+}
+
+namespace {
+struct PendingTiming {
+    const char* name;
+    hipEvent_t start, stop;
+};
+struct TimingState {
+    bool enabled = false;
+    std::vector<PendingTiming> pending;
+    std::vector<hipEvent_t> free_events;
+    std::map<std::string, std::pair<double, uint64_t>> stats;
+};
+TimingState& timing() {
+    static TimingState t;
+    return t;
+}
+hipEvent_t take_event() {
+    TimingState& t = timing();
+    if (!t.free_events.empty()) {
+        hipEvent_t e = t.free_events.back();
+        t.free_events.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+// Waits for the stream and folds every finished (start, stop) pair into the table.
+void resolve_timings() {
+    TimingState& t = timing();
+    if (t.pending.empty()) return;
+    (void)hipStreamSynchronize(ctx().stream);
+    for (const PendingTiming& p : t.pending) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess) {
+            auto& slot = t.stats[p.name];
+            slot.first += ms;
+            slot.second += 1;
+        }
+        t.free_events.push_back(p.start);
+        t.free_events.push_back(p.stop);
+    }
+    t.pending.clear();
+}
+}  // namespace
+
+KernelTimerScope::KernelTimerScope(const char* name) : name_(name) {
+    if (!timing().enabled) return;
+    start_ = take_event();
+    if (start_) (void)hipEventRecord(start_, ctx().stream);
+}
+
+KernelTimerScope::~KernelTimerScope() {
+    if (!start_) return;
+    hipEvent_t stop = take_event();
+    if (!stop) {
+        timing().free_events.push_back(start_);
+        return;
+    }
+    (void)hipEventRecord(stop, ctx().stream);
+    timing().pending.push_back({name_, start_, stop});
 }
 
 }  // namespace ghip
@@ -86,6 +151,11 @@ int granite_hip_shutdown(void) {
     if (c.workspace) (void)hipFree(c.workspace);
     c.workspace = nullptr;
     c.workspace_bytes = 0;
+    ghip::resolve_timings();
+    for (hipEvent_t e : ghip::timing().free_events) (void)hipEventDestroy(e);
+    ghip::timing().free_events.clear();
+    ghip::timing().stats.clear();
+    ghip::timing().enabled = false;
     if (c.own_stream) (void)hipStreamDestroy(c.own_stream);
     c.own_stream = nullptr;
     c.stream = nullptr;
@@ -228,6 +298,50 @@ int granite_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
 }
 
 size_t granite_hip_workspace_bytes(void) { return ctx().workspace_bytes; }
+
+int granite_hip_enable_kernel_timing(int enable) {
+    GHIP_REQUIRE_INIT();
+    ghip::resolve_timings();
+    ghip::timing().enabled = enable != 0;
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_reset_kernel_timing(void) {
+    GHIP_REQUIRE_INIT();
+    ghip::resolve_timings();
+    ghip::timing().stats.clear();
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_get_kernel_timing(const char* kernel_name, double* total_ms,
+                                  uint64_t* dispatches) {
+    GHIP_REQUIRE_INIT();
+    if (!kernel_name || !total_ms || !dispatches) return GRANITE_HIP_ENULL;
+    ghip::resolve_timings();
+    auto it = ghip::timing().stats.find(kernel_name);
+    if (it == ghip::timing().stats.end()) {
+        *total_ms = 0.0;
+        *dispatches = 0;
+        return GRANITE_HIP_OK;
+    }
+    *total_ms = it->second.first;
+    *dispatches = it->second.second;
+    return GRANITE_HIP_OK;
+}
+
+int granite_hip_kernel_timing_names(char* buffer, size_t buffer_bytes) {
+    GHIP_REQUIRE_INIT();
+    if (!buffer || buffer_bytes == 0) return GRANITE_HIP_ENULL;
+    ghip::resolve_timings();
+    std::string all;
+    for (const auto& kv : ghip::timing().stats) {
+        if (!all.empty()) all += ',';
+        all += kv.first;
+    }
+    if (all.size() + 1 > buffer_bytes) return GRANITE_HIP_EINVAL;
+    std::memcpy(buffer, all.c_str(), all.size() + 1);
+    return GRANITE_HIP_OK;
+}
 
 // ---- KV append / gather -------------------------------------------------
 

@@ -40,6 +40,21 @@ int ensure_workspace(size_t bytes);
         if (!::ghip::ctx().initialized) return GRANITE_HIP_ENOTINIT; \
     } while (0)
 
+// Per-kernel GPU timing (MetalCompute::enable_kernel_timing analogue,
+// src/backend/metal/metal_compute.mm:1021-1108).  When enabled, every launch is
+// bracketed by two events on the launch stream; the pairs are resolved into a
+// name -> (milliseconds, dispatches) table when the statistics are read.
+struct KernelTimerScope {
+    explicit KernelTimerScope(const char* name);
+    ~KernelTimerScope();
+    KernelTimerScope(const KernelTimerScope&) = delete;
+    KernelTimerScope& operator=(const KernelTimerScope&) = delete;
+
+  private:
+    const char* name_;
+    hipEvent_t start_ = nullptr;
+};
+
 inline int launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? GRANITE_HIP_OK : static_cast<int>(e);

@@ -361,13 +361,19 @@ int launch_decode(const granite_hip_decode_args& a) {
     dim3 grid(p.max_chunks, p.num_kv_heads * p.q_groups, p.batch);
     dim3 block(kWavesPerWG * kWave);
     hipStream_t st = ctx().stream;
-    if (a.q_dtype == GRANITE_HIP_F32)
-        decode_splitk_kernel<true><<<grid, block, 0, st>>>(p);
-    else
-        decode_splitk_kernel<false><<<grid, block, 0, st>>>(p);
+    {
+        KernelTimerScope timer("decode_splitk");
+        if (a.q_dtype == GRANITE_HIP_F32)
+            decode_splitk_kernel<true><<<grid, block, 0, st>>>(p);
+        else
+            decode_splitk_kernel<false><<<grid, block, 0, st>>>(p);
+    }
     rc = launch_status();
     if (rc != GRANITE_HIP_OK) return rc;
-    decode_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(kHeadDim), 0, st>>>(p);
+    {
+        KernelTimerScope timer("decode_merge");
+        decode_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(kHeadDim), 0, st>>>(p);
+    }
     return launch_status();
 }
 

@@ -165,6 +165,7 @@ int launch_append_typed(const AppendParams& p, int rounding) {
     if (blocks > 65535u * 4) blocks = 65535u * 4;
     dim3 grid(blocks, 2), block(256);
     hipStream_t st = ctx().stream;
+    KernelTimerScope timer("kv_append");
     if (vec) {
         if (rounding == GRANITE_HIP_ROUND_NEAREST)
             kv_append_vec_kernel<SrcT, true><<<grid, block, 0, st>>>(p);
@@ -263,7 +264,10 @@ int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const 
     if (work >= (1ull << 32)) return GRANITE_HIP_EINVAL;
     uint32_t blocks = static_cast<uint32_t>((work + 255) / 256);
     if (blocks > 65535u * 4) blocks = 65535u * 4;
-    kv_gather_kernel<<<dim3(blocks, 2), dim3(256), 0, ctx().stream>>>(p);
+    {
+        KernelTimerScope timer("kv_gather");
+        kv_gather_kernel<<<dim3(blocks, 2), dim3(256), 0, ctx().stream>>>(p);
+    }
     return launch_status();
 }
 

@@ -361,8 +361,11 @@ int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_
     if (!parents || !mask_words) return GRANITE_HIP_ENULL;
     if (num_nodes == 0) return GRANITE_HIP_OK;
     const uint32_t words = (num_nodes + 31) / 32;
-    tree_mask_kernel<<<dim3((num_nodes + 63) / 64), dim3(64), 0, ctx().stream>>>(
-        parents, mask_words, num_nodes, words);
+    {
+        KernelTimerScope timer("tree_mask");
+        tree_mask_kernel<<<dim3((num_nodes + 63) / 64), dim3(64), 0, ctx().stream>>>(
+            parents, mask_words, num_nodes, words);
+    }
     return launch_status();
 }
 
@@ -439,6 +442,7 @@ int launch_attention(const granite_hip_attention_args& a) {
     dim3 grid(q_tiles, a.num_heads), block(kThreads);
     hipStream_t st = ctx().stream;
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
+    KernelTimerScope timer("attention_tiles");
     if (qf32 && of32)
         attention_tiles_kernel<true, true><<<grid, block, 0, st>>>(p);
     else if (qf32 && !of32)

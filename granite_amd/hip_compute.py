@@ -121,6 +121,25 @@ class HipCompute:
     def destroy_event(self, ev: int) -> None:
         check(self.lib.granite_hip_event_destroy(ev), "event_destroy")
 
+    # ---- per-kernel timing (MetalCompute::enable_kernel_timing & co.)
+    def enable_kernel_timing(self, enable: bool) -> None:
+        check(self.lib.granite_hip_enable_kernel_timing(int(enable)), "enable_kernel_timing")
+
+    def reset_kernel_timing(self) -> None:
+        check(self.lib.granite_hip_reset_kernel_timing(), "reset_kernel_timing")
+
+    def get_kernel_timing_stats(self) -> dict:
+        """{kernel name: (total GPU milliseconds, dispatches)}"""
+        buf = C.create_string_buffer(4096)
+        check(self.lib.granite_hip_kernel_timing_names(buf, len(buf)), "kernel_timing_names")
+        stats = {}
+        for name in filter(None, buf.value.decode().split(",")):
+            ms, n = C.c_double(), C.c_uint64()
+            check(self.lib.granite_hip_get_kernel_timing(name.encode(), C.byref(ms), C.byref(n)),
+                  "get_kernel_timing")
+            stats[name] = (ms.value, n.value)
+        return stats
+
     # ---- KV cache
     def kv_cache_append(self, cache_k, cache_v, new_k, new_v, num_kv_heads, head_dim,
                         current_len, new_len, max_seq_len) -> None:
