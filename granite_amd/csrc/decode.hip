@@ -33,6 +33,8 @@
 // (sequence, query head, chunk), and a second kernel merges the chunks.
 //
 // Algorithmic HBM bytes per token of context: 2 (K,V) * num_kv_heads * 128 * 2.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace ghip {
@@ -63,20 +65,6 @@ struct DecodeParams {
     float scale_log2;
 };
 
-__device__ __forceinline__ size_t phys_row(const DecodeParams& p, const int32_t* table,
-                                           uint32_t tok) {
-    if (!table) return tok;
-    uint32_t blk, off;
-    if (p.bs_shift >= 0) {
-        blk = tok >> p.bs_shift;
-        off = tok & (p.block_size - 1);
-    } else {
-        blk = tok / p.block_size;
-        off = tok - blk * p.block_size;
-    }
-    return size_t(table[blk]) * p.block_size + off;
-}
-
 // Token handled by slot j (0..7) of lane group g in the PV contraction.
 __device__ __forceinline__ uint32_t tau(uint32_t g, uint32_t j) {
     return j < 4 ? 4 * g + j : 16 + 4 * g + (j - 4);
@@ -84,9 +72,39 @@ __device__ __forceinline__ uint32_t tau(uint32_t g, uint32_t j) {
 
 __device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
 
-template <bool kQF32>
+// How token positions map to rows of the K/V arrays.
+enum : int { kRowsContiguous = 0, kRowsPagedPow2 = 1, kRowsPagedAny = 2 };
+
+// Physical row of token tok0 + (lane & 31), clamped to the sequence: one table
+// read per lane per tile.  Every other lane fetches the rows it needs from
+// these 32 values with a cross-lane read, so the K/V loads of a tile depend on
+// a single earlier global load instead of one table lookup each.  Branch-free
+// on purpose: a load inside a conditional forces a full wait at the join.
+template <int kRows>
+__device__ __forceinline__ uint32_t tile_row(const DecodeParams& p, const int32_t* table,
+                                             uint32_t tok0, uint32_t lane, uint32_t len) {
+    const uint32_t tok = min(tok0 + (lane & 31), len - 1);
+    if constexpr (kRows == kRowsContiguous) {
+        return tok;
+    } else if constexpr (kRows == kRowsPagedPow2) {
+        return (uint32_t(table[tok >> p.bs_shift]) << p.bs_shift) + (tok & (p.block_size - 1));
+    } else {
+        const uint32_t blk = tok / p.block_size;
+        return uint32_t(table[blk]) * p.block_size + (tok - blk * p.block_size);
+    }
+}
+
+__device__ __forceinline__ uint32_t lane_read(uint32_t v, uint32_t src_lane) {
+    return uint32_t(__builtin_amdgcn_ds_bpermute(int(src_lane << 2), int(v)));
+}
+
+template <bool kQF32, int kRows>
 __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(DecodeParams p) {
-    const uint32_t chunk = blockIdx.x;
+    // Workgroups go to the 8 XCDs round-robin by linear id, and only the first
+    // n_chunks of every (sequence, head) row of the grid carry work.  Rotating
+    // the chunk index per row spreads the live chunks evenly over the XCDs;
+    // without it XCD 0 always gets the odd chunk and finishes last.
+    const uint32_t chunk = (blockIdx.x + blockIdx.y + 3 * blockIdx.z) % gridDim.x;
     const uint32_t kvh = blockIdx.y / p.q_groups;
     const uint32_t qg = blockIdx.y % p.q_groups;
     const uint32_t b = blockIdx.z;
@@ -107,37 +125,44 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
     const bool q_valid = q_in_group < p.group;
     const uint32_t qh = kvh * p.group + (q_valid ? q_in_group : 0);
 
-    const int32_t* table = p.tables ? p.tables + size_t(b) * p.max_blocks : nullptr;
-    const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride;
-    const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride;
+    const int32_t* table =
+        kRows != kRowsContiguous ? p.tables + size_t(b) * p.max_blocks : nullptr;
+    const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride + 8 * g;
+    const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * n;
+
+    // first tile's rows: issued before anything else so the latency overlaps the Q load
+    uint32_t row_cur =
+        tile_row<kRows>(p, table, chunk_start + min(wave, n_tiles - 1) * kTile, lane, len);
 
     // ---- Q as MFMA B operand: lane (n, g), step s holds Q[qh][32s + 8g .. +7]
     half8 bq[4];
-    half8 bq_lo[4];
+    half8 bq_lo[kQF32 ? 4 : 1];
+    {
+        const size_t off = (size_t(b) * p.num_heads + qh) * kHeadDim + 8 * g;
 #pragma unroll
-    for (int s = 0; s < 4; s++) {
-        half8 hi = {0, 0, 0, 0, 0, 0, 0, 0};
-        half8 lo = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (q_valid) {
-            const size_t off = (size_t(b) * p.num_heads + qh) * kHeadDim + 32 * s + 8 * g;
+        for (int s = 0; s < 4; s++) {
             if constexpr (kQF32) {
-                const float* qp = static_cast<const float*>(p.q) + off;
+                const float* qp = static_cast<const float*>(p.q) + off + 32 * s;
                 float4v x0 = *reinterpret_cast<const float4v*>(qp);
                 float4v x1 = *reinterpret_cast<const float4v*>(qp + 4);
                 float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                half8 hi, lo;
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
-                    _Float16 h = static_cast<_Float16>(x[i]);
+                    const float xv = q_valid ? x[i] : 0.0f;
+                    _Float16 h = static_cast<_Float16>(xv);
                     hi[i] = h;
-                    lo[i] = static_cast<_Float16>(x[i] - static_cast<float>(h));
+                    lo[i] = static_cast<_Float16>(xv - static_cast<float>(h));
                 }
+                bq[s] = hi;
+                bq_lo[s] = lo;
             } else {
-                hi = as_half8(*reinterpret_cast<const uint4v*>(
-                    static_cast<const uint16_t*>(p.q) + off));
+                uint4v w = *reinterpret_cast<const uint4v*>(static_cast<const uint16_t*>(p.q) +
+                                                            off + 32 * s);
+                if (!q_valid) w = uint4v{0, 0, 0, 0};
+                bq[s] = as_half8(w);
             }
         }
-        bq[s] = hi;
-        bq_lo[s] = lo;
     }
 
     float m_run = kNegBig;  // running max (log2 domain), identical in the 4 lanes of a column
@@ -149,12 +174,16 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
     for (uint32_t tile = wave; tile < n_tiles; tile += kWavesPerWG) {
         const uint32_t tok0 = chunk_start + tile * kTile;
 
+        // rows of the tile after this one (its table read is in flight during this tile)
+        const uint32_t next = min(tile + kWavesPerWG, n_tiles - 1);
+        const uint32_t row_nxt = tile_row<kRows>(p, table, chunk_start + next * kTile, lane, len);
+
         // ---- K tile: two 16-token sub-tiles, 4 k-steps each
         half8 ka[2][4];
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
-            uint32_t tok = min(tok0 + 16 * sub + n, len - 1);
-            const uint16_t* kp = kbase + phys_row(p, table, tok) * p.tok_stride + 8 * g;
+            const uint32_t row = lane_read(row_cur, 16 * sub + n);
+            const uint16_t* kp = kbase + size_t(row) * p.tok_stride;
 #pragma unroll
             for (int s = 0; s < 4; s++)
                 ka[sub][s] = as_half8(*reinterpret_cast<const uint4v*>(kp + 32 * s));
@@ -163,9 +192,8 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
         uint4v vr[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            uint32_t tok = min(tok0 + tau(g, j), len - 1);
-            const uint16_t* vp = vbase + phys_row(p, table, tok) * p.tok_stride + 8 * n;
-            vr[j] = *reinterpret_cast<const uint4v*>(vp);
+            const uint32_t row = lane_read(row_cur, tau(g, j));
+            vr[j] = *reinterpret_cast<const uint4v*>(vbase + size_t(row) * p.tok_stride);
         }
 
         // ---- S^T = K Q^T
@@ -182,17 +210,20 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
 
         // ---- online softmax; lane (n, g) holds tokens 4g+r and 16+4g+r of column n
         float s[8];
-        float mloc = kNegBig;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            float a = c0[r] * p.scale_log2;
-            float bsc = c1[r] * p.scale_log2;
-            if (tok0 + 4 * g + r >= chunk_end) a = -INFINITY;
-            if (tok0 + 16 + 4 * g + r >= chunk_end) bsc = -INFINITY;
-            s[r] = a;
-            s[4 + r] = bsc;
-            mloc = fmaxf(mloc, fmaxf(a, bsc));
+            s[r] = c0[r] * p.scale_log2;
+            s[4 + r] = c1[r] * p.scale_log2;
         }
+        if (tok0 + kTile > chunk_end) {  // only the last tile of a sequence is ragged
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (tok0 + 4 * g + r >= chunk_end) s[r] = -INFINITY;
+                if (tok0 + 16 + 4 * g + r >= chunk_end) s[4 + r] = -INFINITY;
+            }
+        }
+        float mloc = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                           fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
         mloc = fmaxf(mloc, wave_shfl_xor(mloc, 16));
         mloc = fmaxf(mloc, wave_shfl_xor(mloc, 32));
         const float m_new = fmaxf(m_run, mloc);
@@ -225,6 +256,7 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
             float4v cin = acc[t] * alpha;
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(aw), bp, cin, 0, 0, 0);
         }
+        row_cur = row_nxt;
     }
 
     // ---- reduce the lane-partial sums over the 4 k-groups
@@ -298,7 +330,19 @@ __global__ void __launch_bounds__(kHeadDim) decode_merge_kernel(DecodeParams p) 
 
 }  // namespace
 
-static size_t g_decode_workspace = 0;
+// Split-K chunk used when the caller passes 0.  GRANITE_HIP_DECODE_CHUNK (a
+// multiple of 32) overrides it for tuning runs.
+static uint32_t default_chunk_tokens() {
+    static const uint32_t value = [] {
+        const char* env = std::getenv("GRANITE_HIP_DECODE_CHUNK");
+        if (env) {
+            const long v = std::strtol(env, nullptr, 10);
+            if (v >= kTile && v % kTile == 0 && v <= (1 << 20)) return static_cast<uint32_t>(v);
+        }
+        return 256u;
+    }();
+    return value;
+}
 
 int launch_decode(const granite_hip_decode_args& a) {
     if (!a.q || !a.k_cache || !a.v_cache || !a.out) return GRANITE_HIP_ENULL;
@@ -344,7 +388,7 @@ int launch_decode(const granite_hip_decode_args& a) {
         if (a.fixed_seq_len == 0 || a.fixed_seq_len > p.max_tokens) return GRANITE_HIP_EINVAL;
         p.max_tokens = a.fixed_seq_len;
     }
-    p.chunk_tokens = a.chunk_tokens ? a.chunk_tokens : 256;
+    p.chunk_tokens = a.chunk_tokens ? a.chunk_tokens : default_chunk_tokens();
     if (p.chunk_tokens % kTile != 0) return GRANITE_HIP_EINVAL;
     p.max_chunks = (p.max_tokens + p.chunk_tokens - 1) / p.chunk_tokens;
     p.scale_log2 = a.scale * kLog2e;
@@ -355,7 +399,6 @@ int launch_decode(const granite_hip_decode_args& a) {
     if (rc != GRANITE_HIP_OK) return rc;
     p.part_o = static_cast<float*>(ctx().workspace);
     p.part_ml = p.part_o + slots * kHeadDim;
-    g_decode_workspace = need;
 
     if (p.max_chunks > 65535u * 32 || p.batch > 65535u) return GRANITE_HIP_EINVAL;
     dim3 grid(p.max_chunks, p.num_kv_heads * p.q_groups, p.batch);
@@ -363,10 +406,19 @@ int launch_decode(const granite_hip_decode_args& a) {
     hipStream_t st = ctx().stream;
     {
         KernelTimerScope timer("decode_splitk");
-        if (a.q_dtype == GRANITE_HIP_F32)
-            decode_splitk_kernel<true><<<grid, block, 0, st>>>(p);
-        else
-            decode_splitk_kernel<false><<<grid, block, 0, st>>>(p);
+        const bool qf32 = a.q_dtype == GRANITE_HIP_F32;
+        const int rows = !a.block_tables ? kRowsContiguous
+                                         : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
+#define GHIP_DECODE_CASE(QF32, ROWS)                                   \
+    if (qf32 == QF32 && rows == ROWS)                                  \
+        decode_splitk_kernel<QF32, ROWS><<<grid, block, 0, st>>>(p);
+        GHIP_DECODE_CASE(true, kRowsContiguous)
+        GHIP_DECODE_CASE(true, kRowsPagedPow2)
+        GHIP_DECODE_CASE(true, kRowsPagedAny)
+        GHIP_DECODE_CASE(false, kRowsContiguous)
+        GHIP_DECODE_CASE(false, kRowsPagedPow2)
+        GHIP_DECODE_CASE(false, kRowsPagedAny)
+#undef GHIP_DECODE_CASE
     }
     rc = launch_status();
     if (rc != GRANITE_HIP_OK) return rc;
