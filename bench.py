@@ -130,9 +130,10 @@ def bench_paged_decode(gpu, steps, warmup, cpu):
         "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
         "algorithmic_bytes": nbytes, "flops": c.flops(), "dtype": "f16 K/V, f32 accumulate",
         "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
-        "roofline": roofline("hbm", nbytes, kern["decode_splitk"][0], MEASURED_TRAFFIC["paged_decode"]),
     }
-    res["roofline"]["kernel"] = "decode_splitk_kernel"
+    main_kernel = "decode_stream" if "decode_stream" in kern else "decode_splitk"
+    res["roofline"] = roofline("hbm", nbytes, kern[main_kernel][0], MEASURED_TRAFFIC["paged_decode"])
+    res["roofline"]["kernel"] = main_kernel + "_kernel"
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()

@@ -34,69 +34,13 @@
 //
 // Algorithmic HBM bytes per token of context: 2 (K,V) * num_kv_heads * 128 * 2.
 #include <cstdlib>
+#include <string>
 
 #include "common.h"
+#include "decode_common.h"
 
 namespace ghip {
 namespace {
-
-constexpr int kTile = 32;         // tokens per wave step
-constexpr int kWavesPerWG = 4;
-constexpr float kNegBig = -1.0e30f;
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
-
-struct DecodeParams {
-    const void* q;
-    const uint16_t* k;
-    const uint16_t* v;
-    const int32_t* tables;
-    const int32_t* seq_lens;
-    float* part_o;   // [B, Hq, max_chunks, D]
-    float* part_ml;  // [B, Hq, max_chunks, 2]
-    float* out;
-    float* lse;
-    uint32_t batch, num_heads, num_kv_heads, group, q_groups;
-    uint32_t block_size, max_blocks;
-    int bs_shift;  // log2(block_size) or -1
-    int64_t tok_stride, head_stride;
-    uint32_t max_tokens;  // bound on any sequence length
-    uint32_t chunk_tokens, max_chunks;
-    float scale_log2;
-};
-
-// Token handled by slot j (0..7) of lane group g in the PV contraction.
-__device__ __forceinline__ uint32_t tau(uint32_t g, uint32_t j) {
-    return j < 4 ? 4 * g + j : 16 + 4 * g + (j - 4);
-}
-
-__device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
-
-// How token positions map to rows of the K/V arrays.
-enum : int { kRowsContiguous = 0, kRowsPagedPow2 = 1, kRowsPagedAny = 2 };
-
-// Physical row of token tok0 + (lane & 31), clamped to the sequence: one table
-// read per lane per tile.  Every other lane fetches the rows it needs from
-// these 32 values with a cross-lane read, so the K/V loads of a tile depend on
-// a single earlier global load instead of one table lookup each.  Branch-free
-// on purpose: a load inside a conditional forces a full wait at the join.
-template <int kRows>
-__device__ __forceinline__ uint32_t tile_row(const DecodeParams& p, const int32_t* table,
-                                             uint32_t tok0, uint32_t lane, uint32_t len) {
-    const uint32_t tok = min(tok0 + (lane & 31), len - 1);
-    if constexpr (kRows == kRowsContiguous) {
-        return tok;
-    } else if constexpr (kRows == kRowsPagedPow2) {
-        return (uint32_t(table[tok >> p.bs_shift]) << p.bs_shift) + (tok & (p.block_size - 1));
-    } else {
-        const uint32_t blk = tok / p.block_size;
-        return uint32_t(table[blk]) * p.block_size + (tok - blk * p.block_size);
-    }
-}
-
-__device__ __forceinline__ uint32_t lane_read(uint32_t v, uint32_t src_lane) {
-    return uint32_t(__builtin_amdgcn_ds_bpermute(int(src_lane << 2), int(v)));
-}
 
 template <bool kQF32, int kRows>
 __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(DecodeParams p) {
@@ -344,6 +288,16 @@ static uint32_t default_chunk_tokens() {
     return value;
 }
 
+// GRANITE_HIP_DECODE_MODE=chunk selects the one-workgroup-per-chunk kernel,
+// anything else the persistent one.
+static bool use_stream_kernel() {
+    static const bool value = [] {
+        const char* env = std::getenv("GRANITE_HIP_DECODE_MODE");
+        return !(env && std::string(env) == "chunk");
+    }();
+    return value;
+}
+
 int launch_decode(const granite_hip_decode_args& a) {
     if (!a.q || !a.k_cache || !a.v_cache || !a.out) return GRANITE_HIP_ENULL;
     if (a.head_dim != kHeadDim) return GRANITE_HIP_EINVAL;
@@ -393,6 +347,15 @@ int launch_decode(const granite_hip_decode_args& a) {
     p.max_chunks = (p.max_tokens + p.chunk_tokens - 1) / p.chunk_tokens;
     p.scale_log2 = a.scale * kLog2e;
 
+    const bool qf32 = a.q_dtype == GRANITE_HIP_F32;
+    const int rows = !a.block_tables ? kRowsContiguous
+                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
+    if (use_stream_kernel()) {
+        const uint64_t units = uint64_t(p.batch) * ((p.max_tokens + kTile - 1) / kTile) *
+                               p.num_kv_heads * p.q_groups;
+        if (units < (1ull << 31)) return launch_decode_stream(p, qf32, rows);
+    }
+
     const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;
     const size_t need = slots * (kHeadDim + 2) * sizeof(float);
     int rc = ensure_workspace(need);
@@ -406,9 +369,6 @@ int launch_decode(const granite_hip_decode_args& a) {
     hipStream_t st = ctx().stream;
     {
         KernelTimerScope timer("decode_splitk");
-        const bool qf32 = a.q_dtype == GRANITE_HIP_F32;
-        const int rows = !a.block_tables ? kRowsContiguous
-                                         : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
 #define GHIP_DECODE_CASE(QF32, ROWS)                                   \
     if (qf32 == QF32 && rows == ROWS)                                  \
         decode_splitk_kernel<QF32, ROWS><<<grid, block, 0, st>>>(p);

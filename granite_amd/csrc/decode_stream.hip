@@ -1,0 +1,429 @@
+// Persistent ("stream") form of the decode attention kernel.
+//
+// The context of every (sequence, KV head) is cut into 32-token tiles; all
+// tiles of the batch form one flat list, ordered (sequence, head, tile).  The
+// list is cut into equal contiguous ranges, one per wave, and the grid is one
+// workgroup per compute unit (one wave per SIMD), so every wave streams the same
+// number of K/V bytes and there is no per-chunk workgroup start-up.  (Two
+// workgroups per CU measured slower: the older one wins the memory pipeline and
+// the younger finishes 25 % later.)  A wave that crosses from one (sequence, head) to the next
+// writes a partial (m, l, O) for the part it covered; the merge kernel combines
+// the partials of a (sequence, head), whose positions follow from the same
+// arithmetic.
+//
+// Inside a wave the pipeline is three tiles deep: the block-table rows of tile
+// i+2 and the K/V rows of tile i+1 are in flight while tile i goes through the
+// MFMAs (two register buffers, no LDS, no barriers).  The per-tile math and
+// operand layouts are those of decode.hip.
+#include <cstdlib>
+
+#include "common.h"
+#include "decode_common.h"
+
+namespace ghip {
+namespace {
+
+// One 32-token tile of one (sequence, virtual head).
+struct Cursor {
+    uint32_t b;    // sequence
+    uint32_t vh;   // virtual head = kv_head * q_groups + q_group
+    uint32_t t;    // tile inside the sequence
+    uint32_t nt;   // tiles of sequence b
+    uint32_t len;  // tokens of sequence b
+};
+
+__device__ __forceinline__ uint32_t seq_len_of(const DecodeParams& p, uint32_t b) {
+    uint32_t len = p.seq_lens ? uint32_t(max(p.seq_lens[b], 0)) : p.max_tokens;
+    return min(len, p.max_tokens);
+}
+
+// Next tile in (sequence, head, tile) order; skips empty sequences.  `more`
+// false leaves the cursor where it is (the caller re-reads the last tile
+// instead of running off the end, so no load ever sits inside a branch).
+__device__ __forceinline__ void advance(const DecodeParams& p, Cursor& c, bool more) {
+    if (!more) return;
+    if (++c.t < c.nt) return;
+    c.t = 0;
+    if (++c.vh < p.num_kv_heads * p.q_groups) return;
+    c.vh = 0;
+    do {
+        ++c.b;
+        c.len = c.b < p.batch ? seq_len_of(p, c.b) : kTile;
+        c.nt = (c.len + kTile - 1) / kTile;
+    } while (c.nt == 0 && c.b < p.batch);
+    if (c.b >= p.batch) c.b = p.batch - 1;  // never dereferenced past the end
+}
+
+struct TileRegs {
+    half8 ka[2][4];
+    uint4v vr[8];
+};
+
+template <bool kQF32, int kRows>
+__global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(DecodeParams p) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t n = lane & 15;
+    const uint32_t g = lane >> 4;
+    // wave-uniform by construction; saying so keeps every cursor in scalar registers
+    const uint32_t worker =
+        uint32_t(__builtin_amdgcn_readfirstlane(int(blockIdx.x * kWavesPerWG + wave)));
+
+    // ---- this wave's range of the flat tile list
+    const uint32_t* prefix = p.plan + kPlanHeader;  // prefix[b] = tiles of sequences < b
+    const uint32_t per = p.plan[0];
+    const uint32_t total = p.plan[1];
+    const uint32_t vheads = p.num_kv_heads * p.q_groups;
+    const uint32_t u0 = worker * per;
+    if (u0 >= total) return;
+    const uint32_t n_units = min(per, total - u0);
+
+    // locate u0: largest b with prefix[b] * vheads <= u0
+    Cursor first;
+    {
+        uint32_t lo = 0, hi = p.batch;  // invariant: prefix[lo]*vheads <= u0 < prefix[hi]*vheads
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (prefix[mid] * vheads <= u0) lo = mid; else hi = mid;
+        }
+        first.b = lo;
+        first.nt = prefix[lo + 1] - prefix[lo];
+        first.len = seq_len_of(p, lo);
+        const uint32_t in_seq = u0 - prefix[lo] * vheads;
+        first.vh = in_seq / first.nt;
+        first.t = in_seq - first.vh * first.nt;
+    }
+
+    auto rows_of = [&](const Cursor& c) -> uint32_t {
+        const int32_t* table =
+            kRows != kRowsContiguous ? p.tables + size_t(c.b) * p.max_blocks : nullptr;
+        return tile_row<kRows>(p, table, c.t * kTile, lane, c.len);
+    };
+    auto issue = [&](TileRegs& r, uint32_t rows, const Cursor& c) {
+        const uint32_t kvh = c.vh / p.q_groups;
+        const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride + 8 * g;
+        const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * n;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            const uint32_t row = lane_read(rows, 16 * sub + n);
+            const uint16_t* kp = kbase + size_t(row) * p.tok_stride;
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                r.ka[sub][s] = as_half8(*reinterpret_cast<const uint4v*>(kp + 32 * s));
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t row = lane_read(rows, tau(g, j));
+            r.vr[j] = *reinterpret_cast<const uint4v*>(vbase + size_t(row) * p.tok_stride);
+        }
+    };
+
+    half8 bq[4];
+    half8 bq_lo[kQF32 ? 4 : 1];
+    auto load_q = [&](const Cursor& c) {
+        const uint32_t kvh = c.vh / p.q_groups, qg = c.vh % p.q_groups;
+        const uint32_t q_in_group = qg * 16 + n;
+        const bool q_valid = q_in_group < p.group;
+        const uint32_t qh = kvh * p.group + (q_valid ? q_in_group : 0);
+        const size_t off = (size_t(c.b) * p.num_heads + qh) * kHeadDim + 8 * g;
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            if constexpr (kQF32) {
+                const float* qp = static_cast<const float*>(p.q) + off + 32 * s;
+                float4v x0 = *reinterpret_cast<const float4v*>(qp);
+                float4v x1 = *reinterpret_cast<const float4v*>(qp + 4);
+                float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                half8 hi, lo;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float xv = q_valid ? x[i] : 0.0f;
+                    _Float16 h = static_cast<_Float16>(xv);
+                    hi[i] = h;
+                    lo[i] = static_cast<_Float16>(xv - static_cast<float>(h));
+                }
+                bq[s] = hi;
+                bq_lo[s] = lo;
+            } else {
+                uint4v w = *reinterpret_cast<const uint4v*>(static_cast<const uint16_t*>(p.q) +
+                                                            off + 32 * s);
+                if (!q_valid) w = uint4v{0, 0, 0, 0};
+                bq[s] = as_half8(w);
+            }
+        }
+    };
+
+    float m_run = kNegBig, l_run = 0.0f;
+    float4v acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[t] = float4v{0, 0, 0, 0};
+
+    auto compute = [&](const TileRegs& r, const Cursor& c) {
+        const uint32_t tok0 = c.t * kTile;
+        float4v c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], bq[s], c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], bq[s], c1, 0, 0, 0);
+            if constexpr (kQF32) {
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], bq_lo[s], c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], bq_lo[s], c1, 0, 0, 0);
+            }
+        }
+        float s[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            s[i] = c0[i] * p.scale_log2;
+            s[4 + i] = c1[i] * p.scale_log2;
+        }
+        if (tok0 + kTile > c.len) {  // ragged last tile of a sequence
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (tok0 + 4 * g + i >= c.len) s[i] = -INFINITY;
+                if (tok0 + 16 + 4 * g + i >= c.len) s[4 + i] = -INFINITY;
+            }
+        }
+        float mloc = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                           fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        mloc = fmaxf(mloc, wave_shfl_xor(mloc, 16));
+        mloc = fmaxf(mloc, wave_shfl_xor(mloc, 32));
+        const float m_new = fmaxf(m_run, mloc);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.0f, pj[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            pj[j] = fast_exp2(s[j] - m_new);
+            psum += pj[j];
+        }
+        l_run = l_run * alpha + psum;
+        uint4v bpw;
+        bpw.x = pack_f16x2(pj[0], pj[1]);
+        bpw.y = pack_f16x2(pj[2], pj[3]);
+        bpw.z = pack_f16x2(pj[4], pj[5]);
+        bpw.w = pack_f16x2(pj[6], pj[7]);
+        const half8 bp = as_half8(bpw);
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+            uint4v aw;
+            aw.x = __builtin_amdgcn_perm(r.vr[1][t >> 1], r.vr[0][t >> 1], sel);
+            aw.y = __builtin_amdgcn_perm(r.vr[3][t >> 1], r.vr[2][t >> 1], sel);
+            aw.z = __builtin_amdgcn_perm(r.vr[5][t >> 1], r.vr[4][t >> 1], sel);
+            aw.w = __builtin_amdgcn_perm(r.vr[7][t >> 1], r.vr[6][t >> 1], sel);
+            float4v cin = acc[t] * alpha;
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(aw), bp, cin, 0, 0, 0);
+        }
+    };
+
+    // Writes the partial of the (sequence, head) the cursor is in and clears the state.
+    auto flush = [&](const Cursor& c) {
+        float l = l_run;
+        l += wave_shfl_xor(l, 16);
+        l += wave_shfl_xor(l, 32);
+        const uint32_t kvh = c.vh / p.q_groups, qg = c.vh % p.q_groups;
+        const uint32_t q_in_group = qg * 16 + n;
+        if (q_in_group < p.group) {
+            // slot = this worker's rank among the workers that touch (b, vh)
+            const uint32_t u_start = (prefix[c.b] * vheads) + c.vh * c.nt;
+            const uint32_t slot = worker - u_start / per;
+            const size_t head = size_t(c.b) * p.num_heads + kvh * p.group + q_in_group;
+            const size_t at = head * p.max_chunks + slot;
+            float* po = p.part_o + at * kHeadDim + 32 * g;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float4v w;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int e = 4 * i + k;  // d = 32g + e  <->  acc[e % 8][e / 8]
+                    w[k] = acc[e & 7][e >> 3];
+                }
+                *reinterpret_cast<float4v*>(po + 4 * i) = w;
+            }
+            if (g == 0) {
+                p.part_ml[at * 2 + 0] = m_run;
+                p.part_ml[at * 2 + 1] = l;
+            }
+        }
+        m_run = kNegBig;
+        l_run = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[t] = float4v{0, 0, 0, 0};
+    };
+
+    // ---- three-stage pipeline over the wave's tiles
+    Cursor cc = first;  // tile being computed
+    Cursor cl = first;  // tile whose K/V rows are requested next
+    Cursor cr = first;  // tile whose block-table rows are requested next
+    TileRegs ra, rb;
+
+    uint32_t rows_a = rows_of(cr);
+    advance(p, cr, 1 < n_units);
+    uint32_t rows_b = rows_of(cr);
+    advance(p, cr, 2 < n_units);
+    issue(ra, rows_a, cl);
+    advance(p, cl, 1 < n_units);
+    load_q(cc);
+
+    for (uint32_t i = 0; i < n_units; i += 2) {
+        // tile i+1 (or tile i again at the very end) into buffer B
+        issue(rb, rows_b, cl);
+        advance(p, cl, i + 2 < n_units);
+        rows_a = rows_of(cr);
+        advance(p, cr, i + 3 < n_units);
+
+        compute(ra, cc);
+        {
+            const bool last = i + 1 >= n_units;
+            const bool seg_end = last || cc.t + 1 == cc.nt;
+            const Cursor done = cc;
+            advance(p, cc, !last);
+            if (seg_end) {
+                flush(done);
+                if (!last) load_q(cc);
+            }
+            if (last) break;
+        }
+
+        issue(ra, rows_a, cl);
+        advance(p, cl, i + 3 < n_units);
+        rows_b = rows_of(cr);
+        advance(p, cr, i + 4 < n_units);
+
+        compute(rb, cc);
+        {
+            const bool last = i + 2 >= n_units;
+            const bool seg_end = last || cc.t + 1 == cc.nt;
+            const Cursor done = cc;
+            advance(p, cc, !last);
+            if (seg_end) {
+                flush(done);
+                if (!last) load_q(cc);
+            }
+        }
+    }
+}
+
+// Tiles per sequence, their exclusive prefix sums and the per-wave share of the
+// flat tile list.  One workgroup; the batch is walked in strides of 256.
+__global__ void __launch_bounds__(256) decode_plan_kernel(DecodeParams p, uint32_t workers,
+                                                          uint32_t min_per) {
+    __shared__ uint32_t s_sum[256];
+    __shared__ uint32_t s_base;
+    uint32_t* plan = p.plan;
+    uint32_t* prefix = plan + kPlanHeader;
+    if (threadIdx.x == 0) s_base = 0;
+    __syncthreads();
+    for (uint32_t b0 = 0; b0 < p.batch; b0 += 256) {
+        const uint32_t b = b0 + threadIdx.x;
+        const uint32_t nt = b < p.batch ? (seq_len_of(p, b) + kTile - 1) / kTile : 0;
+        s_sum[threadIdx.x] = nt;
+        __syncthreads();
+        for (uint32_t off = 1; off < 256; off <<= 1) {  // inclusive scan
+            const uint32_t v = threadIdx.x >= off ? s_sum[threadIdx.x - off] : 0;
+            __syncthreads();
+            s_sum[threadIdx.x] += v;
+            __syncthreads();
+        }
+        const uint32_t base = s_base;
+        if (b < p.batch) prefix[b] = base + s_sum[threadIdx.x] - nt;
+        __syncthreads();
+        if (threadIdx.x == 255) s_base = base + s_sum[255];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const uint32_t tiles = s_base;
+        prefix[p.batch] = tiles;
+        const uint32_t total = tiles * p.num_kv_heads * p.q_groups;
+        uint32_t per = (total + workers - 1) / workers;
+        per = max(per, min_per);
+        plan[0] = per;
+        plan[1] = total;
+    }
+}
+
+// Merges the partials of one (sequence, query head): the workers that touched
+// it are consecutive, first = u_start / per, last = (u_end - 1) / per.
+__global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodeParams p) {
+    const uint32_t qh = blockIdx.x;
+    const uint32_t b = blockIdx.y;
+    const uint32_t* prefix = p.plan + kPlanHeader;
+    const uint32_t nt = prefix[b + 1] - prefix[b];
+    if (nt == 0) return;  // empty sequence: output untouched
+    const uint32_t per = p.plan[0];
+    const uint32_t vheads = p.num_kv_heads * p.q_groups;
+    const uint32_t kvh = qh / p.group, qg = (qh % p.group) / 16;
+    const uint32_t vh = kvh * p.q_groups + qg;
+    const uint32_t u_start = prefix[b] * vheads + vh * nt;
+    const uint32_t n_parts = (u_start + nt - 1) / per - u_start / per + 1;
+    const size_t head = size_t(b) * p.num_heads + qh;
+    const float* ml = p.part_ml + head * p.max_chunks * 2;
+    const float* po = p.part_o + head * p.max_chunks * kHeadDim;
+    const uint32_t d = threadIdx.x;
+
+    float mx = kNegBig;
+    for (uint32_t c = 0; c < n_parts; c++) mx = fmaxf(mx, ml[2 * c]);
+    float o = 0.0f, l = 0.0f;
+    for (uint32_t c = 0; c < n_parts; c++) {
+        const float f = fast_exp2(ml[2 * c] - mx);
+        l += ml[2 * c + 1] * f;
+        o += po[size_t(c) * kHeadDim + d] * f;
+    }
+    p.out[head * kHeadDim + d] = o / l;
+    if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
+}
+
+}  // namespace
+
+int launch_decode_stream(DecodeParams p, bool q_f32, int rows) {
+    // Workers: one wave per SIMD on every CU.
+    const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
+    const uint32_t wgs = cus;
+    const uint32_t workers = wgs * kWavesPerWG;
+    // Smallest range a wave may get: it bounds the partial slots per (sequence, head) to
+    // about 32 however short the batch is, and is never above chunk_tokens.
+    const uint32_t max_tiles = (p.max_tokens + kTile - 1) / kTile;
+    const uint32_t min_per = min(max(p.chunk_tokens / kTile, 1u), max((max_tiles + 31) / 32, 1u));
+    p.max_chunks = (max_tiles + min_per - 1) / min_per + 2;  // partial slots per (sequence, head)
+
+    const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;
+    const size_t plan_words = kPlanHeader + size_t(p.batch) + 1;
+    const size_t plan_bytes = (plan_words * sizeof(uint32_t) + 255) & ~size_t(255);
+    const size_t need = plan_bytes + slots * (kHeadDim + 2) * sizeof(float);
+    int rc = ensure_workspace(need);
+    if (rc != GRANITE_HIP_OK) return rc;
+    char* ws = static_cast<char*>(ctx().workspace);
+    p.plan = reinterpret_cast<uint32_t*>(ws);
+    p.part_o = reinterpret_cast<float*>(ws + plan_bytes);
+    p.part_ml = p.part_o + slots * kHeadDim;
+
+    hipStream_t st = ctx().stream;
+    {
+        KernelTimerScope timer("decode_plan");
+        decode_plan_kernel<<<dim3(1), dim3(256), 0, st>>>(p, workers, min_per);
+    }
+    rc = launch_status();
+    if (rc != GRANITE_HIP_OK) return rc;
+    {
+        KernelTimerScope timer("decode_stream");
+        dim3 grid(wgs), block(kWavesPerWG * kWave);
+#define GHIP_STREAM_CASE(QF32, ROWS)                               \
+    if (q_f32 == QF32 && rows == ROWS)                             \
+        decode_stream_kernel<QF32, ROWS><<<grid, block, 0, st>>>(p);
+        GHIP_STREAM_CASE(true, kRowsContiguous)
+        GHIP_STREAM_CASE(true, kRowsPagedPow2)
+        GHIP_STREAM_CASE(true, kRowsPagedAny)
+        GHIP_STREAM_CASE(false, kRowsContiguous)
+        GHIP_STREAM_CASE(false, kRowsPagedPow2)
+        GHIP_STREAM_CASE(false, kRowsPagedAny)
+#undef GHIP_STREAM_CASE
+    }
+    rc = launch_status();
+    if (rc != GRANITE_HIP_OK) return rc;
+    {
+        KernelTimerScope timer("decode_merge");
+        decode_stream_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(kHeadDim), 0, st>>>(p);
+    }
+    return launch_status();
+}
+
+}  // namespace ghip
