@@ -11,13 +11,12 @@
 // tree: cache keys visible, tree key j visible iff j is q or an ancestor).
 //
 // Structure.  grid = (query tiles of 128 rows, query heads); 4 waves, each
-// owning 32 query rows.  Keys are walked in tiles of 64: the workgroup copies
-// the K tile (as is) and the V tile (transposed, token order permuted) into
-// LDS, then every wave computes, with v_mfma_f32_32x32x16_f16,
+// owning 32 query rows.  Keys are walked in tiles of 64.  Per tile every wave
+// computes, with v_mfma_f32_32x32x16_f16,
 //
 //   S^T[key, q]  = K[key, :] . Q[q, :]          (A = K from LDS, B = Q in VGPRs)
-//   online softmax in the result layout: a lane owns one query row and 32 of
-//   the 64 keys, so max/sum are in-lane plus one cross-half shuffle
+//   softmax in the result layout: a lane owns one query row and 32 of the 64
+//   keys, so max/sum are in-lane plus one cross-half shuffle
 //   O^T[d, q]   += V^T[d, key] . P^T[key, q]    (A = V^T from LDS, B = P in VGPRs)
 //
 // Computing the transposed products makes the softmax output of the first
@@ -25,8 +24,22 @@
 // each 16-key group are stored in LDS in the order 8g + 4a + b for key
 // 8a + 4g + b (a, g in {0,1}, b in 0..3).
 //
-// The next tile is fetched from global memory into registers while the
-// current one is being multiplied (one LDS buffer, two barriers per tile).
+// Data movement.  K/V tiles go global -> registers -> LDS, two LDS buffers,
+// one barrier per tile: while tile i is being multiplied, tile i+1 is written
+// to the other buffer, tile i+2 is in flight from HBM and the block-table rows
+// of tile i+3 are being fetched.  K is stored as it lies in memory (row pitch
+// 136 halves); V is stored transposed, V^T[d][key], through an in-register
+// 4x8 transpose (v_perm_b32).  The V^T rows are kept in the order
+// row = 16 * (d % 8) + d / 8 and the thread -> key-quad assignment swaps two
+// index bits, which together make both the 8-byte transposed writes and the
+// 16-byte operand reads free of LDS bank conflicts; as a side effect each lane
+// ends up with runs of 8 consecutive output elements.
+//
+// Softmax rescaling is lazy: probabilities are taken relative to a per-row
+// reference maximum that is only moved (and O, l rescaled) when the row
+// maximum of a tile exceeds it by more than 2^8.  Results are identical up to
+// rounding, P stays inside half range, and the accumulators are left alone in
+// almost every tile.
 //
 // Algorithmic work: 4 * D flops per visible (query, key) pair.
 #include "common.h"
@@ -39,9 +52,15 @@ constexpr int kBN = 64;        // keys per tile
 constexpr int kThreads = 256;  // 4 waves
 constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
 constexpr int kVPitch = kBN + 8;       // halves per V^T row in LDS
+constexpr int kKTileHalves = kBN * kKPitch;
+constexpr int kVTileHalves = kHeadDim * kVPitch;
+constexpr size_t kLdsBytes = 2 * size_t(kKTileHalves + kVTileHalves) * sizeof(uint16_t);
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kRescaleSlack = 8.0f;  // log2 of how far a probability may exceed 1
+
+enum : int { kRowsContiguous = 0, kRowsPagedPow2 = 1, kRowsPagedAny = 2 };
 
 struct AttnParams {
     const void* q;
@@ -67,31 +86,32 @@ struct AttnParams {
 
 __device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
 
-__device__ __forceinline__ size_t phys_row(const AttnParams& p, uint32_t tok) {
-    if (!p.table) return tok;
-    uint32_t blk, off;
-    if (p.bs_shift >= 0) {
-        blk = tok >> p.bs_shift;
-        off = tok & (p.block_size - 1);
+// Row of the K/V array that holds key `idx`: of the cache segment (through the
+// block table when paged) or, with `extra`, of the extra segment (row = idx).
+// Branch-free on purpose: a load inside a conditional makes the compiler wait
+// for every outstanding load at the join, which would serialise the pipeline.
+template <int kRows>
+__device__ __forceinline__ uint32_t key_row(const AttnParams& p, uint32_t idx, bool extra) {
+    if constexpr (kRows == kRowsContiguous) {
+        return idx;
     } else {
-        blk = tok / p.block_size;
-        off = tok - blk * p.block_size;
+        const uint32_t t = extra ? 0u : idx;  // always a valid table position
+        uint32_t row;
+        if constexpr (kRows == kRowsPagedPow2) {
+            row = (uint32_t(p.table[t >> p.bs_shift]) << p.bs_shift) + (t & (p.block_size - 1));
+        } else {
+            const uint32_t blk = t / p.block_size;
+            row = uint32_t(p.table[blk]) * p.block_size + (t - blk * p.block_size);
+        }
+        return extra ? idx : row;
     }
-    return size_t(p.table[blk]) * p.block_size + off;
 }
 
-// Row pointer (head kvh) of key `idx` of segment A (cache) or B (extra).
-__device__ __forceinline__ const uint16_t* key_row(const AttnParams& p, const uint16_t* base_a,
-                                                   const uint16_t* base_b, bool seg_b,
-                                                   uint32_t idx) {
-    if (seg_b) return base_b + size_t(idx) * kHeadDim;
-    return base_a + phys_row(p, idx) * p.a_tok_stride;
-}
-
-template <bool kQF32, bool kOutF32>
-__global__ void __launch_bounds__(kThreads) attention_tiles_kernel(AttnParams p) {
-    __shared__ __attribute__((aligned(16))) uint16_t s_k[kBN * kKPitch];
-    __shared__ __attribute__((aligned(16))) uint16_t s_vt[kHeadDim * kVPitch];
+template <bool kQF32, bool kOutF32, int kRows>
+__global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
+    uint16_t* const s_k0 = s_mem;
+    uint16_t* const s_vt0 = s_mem + 2 * kKTileHalves;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
@@ -153,63 +173,92 @@ __global__ void __launch_bounds__(kThreads) attention_tiles_kernel(AttnParams p)
         }
     }
 
-    // tree mask row of this lane's query (tree mode keeps <= 2 words in registers
-    // per tile; rows are read from global memory per tile)
     const uint32_t* mask_row =
         p.tree_mask ? p.tree_mask + size_t(min(q_row, p.extra_len - 1)) * p.mask_words : nullptr;
 
-    float m_run = kNegBig;
-    float l_run = 0.0f;
+    float m_ref = kNegBig;  // reference maximum (log2 domain) the probabilities are relative to
+    float l_run = 0.0f;     // lane-partial sum (the two k-groups are added at the end)
     float16v oacc[4];
 #pragma unroll
     for (int t = 0; t < 4; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[t][r] = 0.0f;
 
-    // ---- global -> register staging of one K/V tile
-    const uint32_t ld_chunk = tid & 15;  // 16-byte column of the 256-byte row
-    const uint32_t ld_row = tid >> 4;    // 0..15
+    // ---- tile staging: which rows this thread moves
+    const uint32_t ld_c = tid & 15;  // 16-byte column of the 256-byte row
+    const uint32_t ld_r = tid >> 4;  // 0..15
+    // V: key quad with the two low index bits swapped (see the header comment)
+    const uint32_t v_quad = 4 * (ld_r >> 2) + 2 * (ld_r & 1) + ((ld_r >> 1) & 1);
+    const uint32_t v_col = 16 * (ld_r >> 2) + 8 * ((ld_r >> 1) & 1) + 4 * (ld_r & 1);
+
+    struct TileRows {
+        uint32_t k[4];  // rows of keys ld_r + 16 i
+        uint32_t v[4];  // rows of keys 4 v_quad + i
+    };
     uint4v kreg[4], vreg[4];
 
-    auto load_tile = [&](uint32_t it) {
+    auto tile_rows = [&](uint32_t it, TileRows& r) {
+        it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
-        const uint32_t seg_len = seg_b ? len_b : len_a;
+        const uint32_t last = (seg_b ? len_b : len_a) - 1;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t kk = min(key0 + ld_row + 16 * i, seg_len - 1);
-            kreg[i] = *reinterpret_cast<const uint4v*>(key_row(p, ka_base, kb_base, seg_b, kk) +
-                                                       8 * ld_chunk);
-            const uint32_t vk = min(key0 + 4 * ld_row + i, seg_len - 1);
-            vreg[i] = *reinterpret_cast<const uint4v*>(key_row(p, va_base, vb_base, seg_b, vk) +
-                                                       8 * ld_chunk);
+            const uint32_t kk = min(key0 + ld_r + 16 * i, last);
+            const uint32_t vk = min(key0 + 4 * v_quad + i, last);
+            r.k[i] = key_row<kRows>(p, kk, seg_b);
+            r.v[i] = key_row<kRows>(p, vk, seg_b);
         }
     };
-
-    auto store_tile = [&]() {
+    auto load_tile = [&](uint32_t it, const TileRows& r) {
+        it = min(it, n_tiles - 1);
+        const bool seg_b = it >= tiles_a;
+        const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
+        const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
+        const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            kreg[i] = *reinterpret_cast<const uint4v*>(kb + int64_t(r.k[i]) * stride);
+            vreg[i] = *reinterpret_cast<const uint4v*>(vb + int64_t(r.v[i]) * stride);
+        }
+    };
+    auto store_tile = [&](uint32_t buf) {
+        uint16_t* sk = s_k0 + buf * kKTileHalves;
+        uint16_t* sv = s_vt0 + buf * kVTileHalves;
 #pragma unroll
         for (int i = 0; i < 4; i++)
-            *reinterpret_cast<uint4v*>(&s_k[(ld_row + 16 * i) * kKPitch + 8 * ld_chunk]) = kreg[i];
-        // V: 4 keys x 8 d  ->  8 rows (d) of 4 keys; column = permuted key position
-        const uint32_t kq = ld_row;  // key quad 0..15 : keys 4kq .. 4kq+3
-        const uint32_t col = 16 * (kq >> 2) + 8 * (kq & 1) + 4 * ((kq >> 1) & 1);
+            *reinterpret_cast<uint4v*>(&sk[(ld_r + 16 * i) * kKPitch + 8 * ld_c]) = kreg[i];
+        // V: 4 keys x 8 d  ->  8 rows of 4 keys; row of d = 8 ld_c + t is 16 t + ld_c
 #pragma unroll
         for (int t = 0; t < 8; t++) {
             const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
             uint2v w;
             w.x = __builtin_amdgcn_perm(vreg[1][t >> 1], vreg[0][t >> 1], sel);
             w.y = __builtin_amdgcn_perm(vreg[3][t >> 1], vreg[2][t >> 1], sel);
-            *reinterpret_cast<uint2v*>(&s_vt[(8 * ld_chunk + t) * kVPitch + col]) = w;
+            *reinterpret_cast<uint2v*>(&sv[(16 * t + ld_c) * kVPitch + v_col]) = w;
         }
     };
 
-    if (n_tiles > 0) load_tile(0);
+    if (n_tiles == 0) return;  // nothing visible (not reachable through the C ABI checks)
+
+    // ---- prologue: tile 0 in LDS, tile 1 in flight, rows of tile 2 requested
+    TileRows rows;
+    tile_rows(0, rows);
+    load_tile(0, rows);
+    tile_rows(1, rows);
+    store_tile(0);
+    load_tile(1, rows);
+    tile_rows(2, rows);
+    __syncthreads();
 
     for (uint32_t it = 0; it < n_tiles; it++) {
-        __syncthreads();
-        store_tile();
-        __syncthreads();
-        if (it + 1 < n_tiles) load_tile(it + 1);
+        const uint32_t buf = it & 1;
+        // Unconditional (indices clamp at the last tile): loads inside a branch would
+        // force a full wait at the join.  The extra store after the last tile goes to the
+        // buffer nobody reads any more.
+        store_tile(buf ^ 1);      // tile it+1 (arrived during the previous tile)
+        load_tile(it + 2, rows);  // tile it+2 flies during this tile's math
+        tile_rows(it + 3, rows);
 
         const bool seg_b = it >= tiles_a;
         const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
@@ -220,97 +269,107 @@ __global__ void __launch_bounds__(kThreads) attention_tiles_kernel(AttnParams p)
             const uint32_t q_last_wave = min(q0 + 32, p.seq_q) - 1;
             if (key0 > p.start_pos + q_last_wave) compute = false;
         }
-        if (!compute) continue;
+        if (compute) {
+            const uint16_t* sk = s_k0 + buf * kKTileHalves;
+            const uint16_t* sv = s_vt0 + buf * kVTileHalves;
 
-        // ---- S^T for the two 32-key sub-tiles
-        float16v sacc[2];
-#pragma unroll
-        for (int sub = 0; sub < 2; sub++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) sacc[sub][r] = 0.0f;
-            const uint16_t* krow = &s_k[(32 * sub + n) * kKPitch + 8 * g];
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const half8 a = as_half8(*reinterpret_cast<const uint4v*>(krow + 16 * s));
-                sacc[sub] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[s], sacc[sub], 0, 0, 0);
-                if constexpr (kQF32)
-                    sacc[sub] =
-                        __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[s], sacc[sub], 0, 0, 0);
-            }
-        }
-
-        // ---- masks (only on tiles that need them)
-        const bool partial = key0 + kBN > seg_len;
-        const bool diagonal = p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !seg_b &&
-                              key0 + kBN - 1 > p.start_pos + q0;
-        const bool tree = p.mask_mode == GRANITE_HIP_MASK_TREE && seg_b;
-        if (partial || diagonal || tree) {
-            uint32_t mw0 = 0xFFFFFFFFu, mw1 = 0xFFFFFFFFu;
-            if (tree) {
-                const uint32_t w = key0 >> 5;
-                mw0 = w < p.mask_words ? mask_row[w] : 0u;
-                mw1 = w + 1 < p.mask_words ? mask_row[w + 1] : 0u;
-            }
-            const uint32_t limit = diagonal ? min(seg_len, p.start_pos + q_row + 1) : seg_len;
+            // ---- S^T for the two 32-key sub-tiles
+            float16v sacc[2];
 #pragma unroll
             for (int sub = 0; sub < 2; sub++) {
-                const uint32_t mw = sub ? mw1 : mw0;
+                const uint16_t* krow = &sk[(32 * sub + n) * kKPitch + 8 * g];
+                float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t kin = 8 * (r >> 2) + 4 * g + (r & 3);  // key inside sub-tile
-                    const bool vis = (key0 + 32 * sub + kin < limit) && ((mw >> kin) & 1u);
-                    if (!vis) sacc[sub][r] = -INFINITY;
+                for (int s = 0; s < 8; s++) {
+                    const half8 a = as_half8(*reinterpret_cast<const uint4v*>(krow + 16 * s));
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[s], c, 0, 0, 0);
+                    if constexpr (kQF32)
+                        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[s], c, 0, 0, 0);
+                }
+                sacc[sub] = c;
+            }
+
+            // ---- masks (only on tiles that need them)
+            const bool partial = key0 + kBN > seg_len;
+            const bool diagonal = p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !seg_b &&
+                                  key0 + kBN - 1 > p.start_pos + q0;
+            const bool tree = p.mask_mode == GRANITE_HIP_MASK_TREE && seg_b;
+            if (partial || diagonal || tree) {
+                uint32_t mw0 = 0xFFFFFFFFu, mw1 = 0xFFFFFFFFu;
+                if (tree) {
+                    const uint32_t w = key0 >> 5;
+                    mw0 = w < p.mask_words ? mask_row[w] : 0u;
+                    mw1 = w + 1 < p.mask_words ? mask_row[w + 1] : 0u;
+                }
+                const uint32_t limit = diagonal ? min(seg_len, p.start_pos + q_row + 1) : seg_len;
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++) {
+                    const uint32_t mw = sub ? mw1 : mw0;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const uint32_t kin = 8 * (r >> 2) + 4 * g + (r & 3);  // key in sub-tile
+                        const bool vis = (key0 + 32 * sub + kin < limit) && ((mw >> kin) & 1u);
+                        if (!vis) sacc[sub][r] = -INFINITY;
+                    }
                 }
             }
-        }
 
-        // ---- online softmax (raw scores; the scale is folded into the exponent)
-        float mraw = -INFINITY;
+            // ---- softmax relative to m_ref; move m_ref only when a row outgrows it
+            float mraw = -INFINITY;
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++)
+            for (int sub = 0; sub < 2; sub++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[sub][r]);
-        mraw = fmaxf(mraw, wave_shfl_xor(mraw, 32));
-        const float m_new = fmaxf(m_run, mraw * p.scale_log2);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.0f;
-        half8 bp[2][2];
+                for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[sub][r]);
+            mraw = fmaxf(mraw, wave_shfl_xor(mraw, 32));
+            const float m_tile = mraw * p.scale_log2;
+            if (__any(m_tile > m_ref + kRescaleSlack)) {
+                const float m_new = fmaxf(m_ref, m_tile);
+                const float alpha = fast_exp2(m_ref - m_new);
+                m_ref = m_new;
+                l_run *= alpha;
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++)
+                for (int t = 0; t < 4; t++)
 #pragma unroll
-            for (int u = 0; u < 2; u++) {
-                float pe[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    pe[j] = fast_exp2(__builtin_fmaf(sacc[sub][8 * u + j], p.scale_log2, -m_new));
-                    psum += pe[j];
-                }
-                uint4v w;
-                w.x = pack_f16x2(pe[0], pe[1]);
-                w.y = pack_f16x2(pe[2], pe[3]);
-                w.z = pack_f16x2(pe[4], pe[5]);
-                w.w = pack_f16x2(pe[6], pe[7]);
-                bp[sub][u] = as_half8(w);
+                    for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
             }
-        l_run = l_run * alpha + psum;
-
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
-            const uint16_t* vrow = &s_vt[(32 * t + n) * kVPitch + 8 * g];
+            float psum = 0.0f;
+            half8 bp[2][2];
 #pragma unroll
             for (int sub = 0; sub < 2; sub++)
 #pragma unroll
                 for (int u = 0; u < 2; u++) {
-                    const half8 a =
-                        as_half8(*reinterpret_cast<const uint4v*>(vrow + 32 * sub + 16 * u));
-                    oacc[t] =
-                        __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp[sub][u], oacc[t], 0, 0, 0);
+                    float pe[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        pe[j] =
+                            fast_exp2(__builtin_fmaf(sacc[sub][8 * u + j], p.scale_log2, -m_ref));
+                        psum += pe[j];
+                    }
+                    uint4v w;
+                    w.x = pack_f16x2(pe[0], pe[1]);
+                    w.y = pack_f16x2(pe[2], pe[3]);
+                    w.z = pack_f16x2(pe[4], pe[5]);
+                    w.w = pack_f16x2(pe[6], pe[7]);
+                    bp[sub][u] = as_half8(w);
                 }
+            l_run += psum;
+
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint16_t* vrow = &sv[(32 * t + n) * kVPitch + 8 * g];
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                    for (int u = 0; u < 2; u++) {
+                        const half8 a =
+                            as_half8(*reinterpret_cast<const uint4v*>(vrow + 32 * sub + 16 * u));
+                        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp[sub][u], oacc[t],
+                                                                         0, 0, 0);
+                    }
+            }
         }
+        __syncthreads();
     }
 
     if (!wave_active) return;
@@ -318,25 +377,31 @@ __global__ void __launch_bounds__(kThreads) attention_tiles_kernel(AttnParams p)
     if (q_row >= p.seq_q) return;
     const float inv_l = 1.0f / l_run;
     const int64_t ooff = int64_t(q_row) * p.out_tok_stride + int64_t(head) * p.out_head_stride;
+    // Accumulator [t][4a + b] is LDS row 32t + 8a + 4g + b, i.e. head-dim element
+    // 64 (a & 1) + 32 g + 8 b + 2 t + (a >> 1): 8 consecutive elements per (a & 1, b).
 #pragma unroll
-    for (int t = 0; t < 4; t++)
+    for (int al = 0; al < 2; al++)
 #pragma unroll
-        for (int a = 0; a < 4; a++) {
-            const uint32_t d = 32 * t + 8 * a + 4 * g;
-            const float x0 = oacc[t][4 * a + 0] * inv_l, x1 = oacc[t][4 * a + 1] * inv_l;
-            const float x2 = oacc[t][4 * a + 2] * inv_l, x3 = oacc[t][4 * a + 3] * inv_l;
+        for (int b = 0; b < 4; b++) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = oacc[e >> 1][4 * (al + 2 * (e & 1)) + b] * inv_l;
+            const uint32_t d = 64 * al + 32 * g + 8 * b;
             if constexpr (kOutF32) {
-                *reinterpret_cast<float4v*>(static_cast<float*>(p.out) + ooff + d) =
-                    float4v{x0, x1, x2, x3};
+                float* op = static_cast<float*>(p.out) + ooff + d;
+                *reinterpret_cast<float4v*>(op) = float4v{x[0], x[1], x[2], x[3]};
+                *reinterpret_cast<float4v*>(op + 4) = float4v{x[4], x[5], x[6], x[7]};
             } else {
-                uint2v w;
-                w.x = pack_f16x2(x0, x1);
-                w.y = pack_f16x2(x2, x3);
-                *reinterpret_cast<uint2v*>(static_cast<uint16_t*>(p.out) + ooff + d) = w;
+                uint4v w;
+                w.x = pack_f16x2(x[0], x[1]);
+                w.y = pack_f16x2(x[2], x[3]);
+                w.z = pack_f16x2(x[4], x[5]);
+                w.w = pack_f16x2(x[6], x[7]);
+                *reinterpret_cast<uint4v*>(static_cast<uint16_t*>(p.out) + ooff + d) = w;
             }
         }
     if (p.lse && g == 0)
-        p.lse[size_t(head) * p.seq_q + q_row] = (m_run + __builtin_amdgcn_logf(l_run)) * kLn2;
+        p.lse[size_t(head) * p.seq_q + q_row] = (m_ref + __builtin_amdgcn_logf(l_run)) * kLn2;
 }
 
 // One thread per node: set own bit, then walk parent pointers
@@ -353,6 +418,27 @@ __global__ void tree_mask_kernel(const int32_t* parents, uint32_t* mask, uint32_
         row[uint32_t(cur) >> 5] |= 1u << (uint32_t(cur) & 31);
         cur = parents[cur];
     }
+}
+
+template <bool kQF32, bool kOutF32, int kRows>
+int launch_tiles(const AttnParams& p, dim3 grid) {
+    auto kernel = attention_tiles_kernel<kQF32, kOutF32, kRows>;
+    static bool configured = false;  // the two LDS buffers exceed the 64 KiB default limit
+    if (!configured) {
+        GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(kLdsBytes)));
+        configured = true;
+    }
+    kernel<<<grid, dim3(kThreads), kLdsBytes, ctx().stream>>>(p);
+    return launch_status();
+}
+
+template <bool kQF32, bool kOutF32>
+int launch_tiles_rows(const AttnParams& p, dim3 grid, int rows) {
+    if (rows == kRowsContiguous) return launch_tiles<kQF32, kOutF32, kRowsContiguous>(p, grid);
+    if (rows == kRowsPagedPow2) return launch_tiles<kQF32, kOutF32, kRowsPagedPow2>(p, grid);
+    return launch_tiles<kQF32, kOutF32, kRowsPagedAny>(p, grid);
 }
 
 }  // namespace
@@ -439,19 +525,15 @@ int launch_attention(const granite_hip_attention_args& a) {
 
     const uint32_t q_tiles = (a.seq_q + kBM - 1) / kBM;
     if (q_tiles > 0x7FFFFFFFu / 2 || a.num_heads > 65535u) return GRANITE_HIP_EINVAL;
-    dim3 grid(q_tiles, a.num_heads), block(kThreads);
-    hipStream_t st = ctx().stream;
+    dim3 grid(q_tiles, a.num_heads);
+    const int rows = !a.block_table ? kRowsContiguous
+                                    : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
     KernelTimerScope timer("attention_tiles");
-    if (qf32 && of32)
-        attention_tiles_kernel<true, true><<<grid, block, 0, st>>>(p);
-    else if (qf32 && !of32)
-        attention_tiles_kernel<true, false><<<grid, block, 0, st>>>(p);
-    else if (!qf32 && of32)
-        attention_tiles_kernel<false, true><<<grid, block, 0, st>>>(p);
-    else
-        attention_tiles_kernel<false, false><<<grid, block, 0, st>>>(p);
-    return launch_status();
+    if (qf32 && of32) return launch_tiles_rows<true, true>(p, grid, rows);
+    if (qf32 && !of32) return launch_tiles_rows<true, false>(p, grid, rows);
+    if (!qf32 && of32) return launch_tiles_rows<false, true>(p, grid, rows);
+    return launch_tiles_rows<false, false>(p, grid, rows);
 }
 
 }  // namespace ghip
