@@ -42,6 +42,8 @@
 // almost every tile.
 //
 // Algorithmic work: 4 * D flops per visible (query, key) pair.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace ghip {
@@ -82,6 +84,11 @@ struct AttnParams {
     int mask_mode;
     uint32_t start_pos, seq_q, num_heads, group;
     float scale_log2;
+    // split-K over the key tiles (gridDim.z > 1): unnormalised partial results
+    float* part_o;   // [split, head, q, D]
+    float* part_ml;  // [split, head, q, 2] = (reference max, sum)
+    void* final_out;
+    int64_t final_tok_stride, final_head_stride;
 };
 
 __device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
@@ -138,7 +145,10 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     const uint32_t len_b = p.extra_len;
     const uint32_t tiles_a = (len_a + kBN - 1) / kBN;
     const uint32_t tiles_b = (len_b + kBN - 1) / kBN;
-    const uint32_t n_tiles = tiles_a + tiles_b;
+    const uint32_t all_tiles = tiles_a + tiles_b;
+    // this workgroup's share of the key tiles when the keys are split over gridDim.z
+    const uint32_t t_begin = uint32_t(uint64_t(all_tiles) * blockIdx.z / gridDim.z);
+    const uint32_t n_tiles = uint32_t(uint64_t(all_tiles) * (blockIdx.z + 1) / gridDim.z);
 
     const uint16_t* ka_base = p.k + size_t(kvh) * p.a_head_stride;
     const uint16_t* va_base = p.v + size_t(kvh) * p.a_head_stride;
@@ -239,19 +249,18 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
     };
 
-    if (n_tiles == 0) return;  // nothing visible (not reachable through the C ABI checks)
-
-    // ---- prologue: tile 0 in LDS, tile 1 in flight, rows of tile 2 requested
+    if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
+    // ---- prologue: first tile in LDS, second in flight, rows of the third requested
     TileRows rows;
-    tile_rows(0, rows);
-    load_tile(0, rows);
-    tile_rows(1, rows);
-    store_tile(0);
-    load_tile(1, rows);
-    tile_rows(2, rows);
+    tile_rows(t_begin, rows);
+    load_tile(t_begin, rows);
+    tile_rows(t_begin + 1, rows);
+    store_tile(t_begin & 1);
+    load_tile(t_begin + 1, rows);
+    tile_rows(t_begin + 2, rows);
     __syncthreads();
 
-    for (uint32_t it = 0; it < n_tiles; it++) {
+    for (uint32_t it = t_begin; it < n_tiles; it++) {
         const uint32_t buf = it & 1;
         // Unconditional (indices clamp at the last tile): loads inside a branch would
         // force a full wait at the join.  The extra store after the last tile goes to the
@@ -371,10 +380,32 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         __syncthreads();
     }
+    }
 
     if (!wave_active) return;
     l_run += wave_shfl_xor(l_run, 32);
     if (q_row >= p.seq_q) return;
+    if (gridDim.z > 1) {
+        // partial result of this key range: O unnormalised, (m_ref, l) beside it
+        const size_t row = (size_t(blockIdx.z) * p.num_heads + head) * p.seq_q + q_row;
+        float* po = p.part_o + row * kHeadDim;
+#pragma unroll
+        for (int al = 0; al < 2; al++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                float x[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[e] = oacc[e >> 1][4 * (al + 2 * (e & 1)) + b];
+                float* op = po + 64 * al + 32 * g + 8 * b;
+                *reinterpret_cast<float4v*>(op) = float4v{x[0], x[1], x[2], x[3]};
+                *reinterpret_cast<float4v*>(op + 4) = float4v{x[4], x[5], x[6], x[7]};
+            }
+        if (g == 0) {
+            p.part_ml[row * 2 + 0] = m_ref;
+            p.part_ml[row * 2 + 1] = l_run;
+        }
+        return;
+    }
     const float inv_l = 1.0f / l_run;
     const int64_t ooff = int64_t(q_row) * p.out_tok_stride + int64_t(head) * p.out_head_stride;
     // Accumulator [t][4a + b] is LDS row 32t + 8a + 4g + b, i.e. head-dim element
@@ -418,6 +449,52 @@ __global__ void tree_mask_kernel(const int32_t* parents, uint32_t* mask, uint32_
         row[uint32_t(cur) >> 5] |= 1u << (uint32_t(cur) & 31);
         cur = parents[cur];
     }
+}
+
+// Combines the split-K partials of 16 query rows of one head: one thread per
+// (row, 8 consecutive head-dim elements).
+template <bool kOutF32>
+__global__ void __launch_bounds__(256) attention_merge_kernel(AttnParams p, uint32_t n_splits) {
+    const uint32_t head = blockIdx.y;
+    const uint32_t q_row = blockIdx.x * 16 + (threadIdx.x >> 4);
+    const uint32_t dc = threadIdx.x & 15;
+    if (q_row >= p.seq_q) return;
+    float mx = kNegBig;
+    for (uint32_t s = 0; s < n_splits; s++) {
+        const size_t row = (size_t(s) * p.num_heads + head) * p.seq_q + q_row;
+        mx = fmaxf(mx, p.part_ml[row * 2]);
+    }
+    float l = 0.0f;
+    float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (uint32_t s = 0; s < n_splits; s++) {
+        const size_t row = (size_t(s) * p.num_heads + head) * p.seq_q + q_row;
+        const float f = fast_exp2(p.part_ml[row * 2] - mx);
+        l += p.part_ml[row * 2 + 1] * f;
+        const float* po = p.part_o + row * kHeadDim + 8 * dc;
+        const float4v a = *reinterpret_cast<const float4v*>(po);
+        const float4v b = *reinterpret_cast<const float4v*>(po + 4);
+        o[0] += a.x * f; o[1] += a.y * f; o[2] += a.z * f; o[3] += a.w * f;
+        o[4] += b.x * f; o[5] += b.y * f; o[6] += b.z * f; o[7] += b.w * f;
+    }
+    const float inv_l = 1.0f / l;
+    const int64_t ooff =
+        int64_t(q_row) * p.final_tok_stride + int64_t(head) * p.final_head_stride + 8 * dc;
+    if constexpr (kOutF32) {
+        float* op = static_cast<float*>(p.final_out) + ooff;
+        *reinterpret_cast<float4v*>(op) =
+            float4v{o[0] * inv_l, o[1] * inv_l, o[2] * inv_l, o[3] * inv_l};
+        *reinterpret_cast<float4v*>(op + 4) =
+            float4v{o[4] * inv_l, o[5] * inv_l, o[6] * inv_l, o[7] * inv_l};
+    } else {
+        uint4v w;
+        w.x = pack_f16x2(o[0] * inv_l, o[1] * inv_l);
+        w.y = pack_f16x2(o[2] * inv_l, o[3] * inv_l);
+        w.z = pack_f16x2(o[4] * inv_l, o[5] * inv_l);
+        w.w = pack_f16x2(o[6] * inv_l, o[7] * inv_l);
+        *reinterpret_cast<uint4v*>(static_cast<uint16_t*>(p.final_out) + ooff) = w;
+    }
+    if (p.lse && dc == 0)
+        p.lse[size_t(head) * p.seq_q + q_row] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
 }
 
 template <bool kQF32, bool kOutF32, int kRows>
@@ -512,28 +589,72 @@ int launch_attention(const granite_hip_attention_args& a) {
         if (!a.parents) return GRANITE_HIP_ENULL;
         if (a.extra_len == 0 || a.seq_q != a.extra_len) return GRANITE_HIP_EINVAL;
         p.mask_words = (a.extra_len + 31) / 32;
-        const size_t need = size_t(a.extra_len) * p.mask_words * sizeof(uint32_t);
-        int rc = ensure_workspace(need);
-        if (rc != GRANITE_HIP_OK) return rc;
-        uint32_t* mask = static_cast<uint32_t*>(ctx().workspace);
-        rc = launch_tree_mask(a.parents, mask, a.extra_len);
-        if (rc != GRANITE_HIP_OK) return rc;
-        p.tree_mask = mask;
     } else if (a.mask_mode != GRANITE_HIP_MASK_NONE) {
         return GRANITE_HIP_EINVAL;
     }
 
     const uint32_t q_tiles = (a.seq_q + kBM - 1) / kBM;
     if (q_tiles > 0x7FFFFFFFu / 2 || a.num_heads > 65535u) return GRANITE_HIP_EINVAL;
-    dim3 grid(q_tiles, a.num_heads);
+
+    // Split the keys over several workgroups when (query tiles x heads) alone cannot
+    // put two workgroups on every CU; every split keeps at least 4 key tiles.
+    uint32_t n_splits = 1;
+    {
+        const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
+        const uint64_t wgs = uint64_t(q_tiles) * a.num_heads;
+        const uint32_t key_tiles = (a.cache_len + kBN - 1) / kBN + (a.extra_len + kBN - 1) / kBN;
+        if (wgs < 2 * cus) {
+            n_splits = uint32_t((2 * cus + wgs - 1) / wgs);
+            n_splits = min(n_splits, max(key_tiles / 4, 1u));
+            n_splits = min(n_splits, 64u);
+        }
+        if (const char* e = std::getenv("GRANITE_HIP_ATTN_SPLITS")) n_splits = max(1, std::atoi(e));
+    }
+    // One scratch request for everything (growing the scratch buffer moves it): the
+    // tree mask first, the split-K partials behind it.
+    const bool tree = a.mask_mode == GRANITE_HIP_MASK_TREE;
+    const size_t mask_bytes =
+        tree ? (size_t(a.extra_len) * p.mask_words * sizeof(uint32_t) + 255) & ~size_t(255) : 0;
+    const size_t rows_total = n_splits > 1 ? size_t(n_splits) * a.num_heads * a.seq_q : 0;
+    const size_t need = mask_bytes + rows_total * (kHeadDim + 2) * sizeof(float);
+    if (need > 0) {
+        int rc = ensure_workspace(need);
+        if (rc != GRANITE_HIP_OK) return rc;
+        char* ws = static_cast<char*>(ctx().workspace);
+        if (tree) {
+            uint32_t* mask = reinterpret_cast<uint32_t*>(ws);
+            rc = launch_tree_mask(a.parents, mask, a.extra_len);
+            if (rc != GRANITE_HIP_OK) return rc;
+            p.tree_mask = mask;
+        }
+        if (n_splits > 1) {
+            p.part_o = reinterpret_cast<float*>(ws + mask_bytes);
+            p.part_ml = p.part_o + rows_total * kHeadDim;
+            p.final_out = a.out;
+            p.final_tok_stride = a.out_tok_stride;
+            p.final_head_stride = a.out_head_stride;
+        }
+    }
+    dim3 grid(q_tiles, a.num_heads, n_splits);
     const int rows = !a.block_table ? kRowsContiguous
                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
-    KernelTimerScope timer("attention_tiles");
-    if (qf32 && of32) return launch_tiles_rows<true, true>(p, grid, rows);
-    if (qf32 && !of32) return launch_tiles_rows<true, false>(p, grid, rows);
-    if (!qf32 && of32) return launch_tiles_rows<false, true>(p, grid, rows);
-    return launch_tiles_rows<false, false>(p, grid, rows);
+    int rc;
+    {
+        KernelTimerScope timer("attention_tiles");
+        if (qf32 && of32) rc = launch_tiles_rows<true, true>(p, grid, rows);
+        else if (qf32 && !of32) rc = launch_tiles_rows<true, false>(p, grid, rows);
+        else if (!qf32 && of32) rc = launch_tiles_rows<false, true>(p, grid, rows);
+        else rc = launch_tiles_rows<false, false>(p, grid, rows);
+    }
+    if (rc != GRANITE_HIP_OK || n_splits == 1) return rc;
+    {
+        KernelTimerScope timer("attention_merge");
+        dim3 mgrid((a.seq_q + 15) / 16, a.num_heads);
+        if (of32) attention_merge_kernel<true><<<mgrid, dim3(256), 0, ctx().stream>>>(p, n_splits);
+        else attention_merge_kernel<false><<<mgrid, dim3(256), 0, ctx().stream>>>(p, n_splits);
+    }
+    return launch_status();
 }
 
 }  // namespace ghip
