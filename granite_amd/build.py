@@ -79,10 +79,7 @@ def build_hip_library(jobs: int = 4, extra_flags: list[str] | None = None) -> Pa
 def build_host_layer() -> list[Path]:
     """Compile the C++20 host layer (backend, compute API, operator, KV state)
     and its test programs with g++; they bind libgranite_hip.so through the C ABI."""
-    mk = HOST / "Makefile"
-    if not mk.exists():
-        return []
-    _run(["make", "-C", str(HOST), "-j4"])
+    _run(["make", "-C", str(HOST), "-B", "-j4"])
     return sorted(BINDIR.glob("*"))
 
 
@@ -93,8 +90,8 @@ def build_oracle() -> None:
 
 def build_all() -> None:
     build_hip_library()
+    build_oracle()  # the host layer's test programs link it as their checker
     build_host_layer()
-    build_oracle()
 
 
 if __name__ == "__main__":

@@ -1,0 +1,150 @@
+// HipAttentionOp: OpType::ScaledDotProductAttention on BackendType::HIP.
+//
+// Stands where MetalAttentionOp stands in the reference
+// (src/operators/metal/metal_operators.mm:1226-1320): inputs Q, K, V, one output
+// shaped like Q, attributes `scale` (default 1/sqrt(D)) and `start_pos`
+// (default 0), key k visible to query q iff k <= q + start_pos
+// (metal_operators.mm:640-641).  Unlike that operator it works on the device
+// buffers in place (no map/copy round trip) and accepts head dimensions:
+//   Q, out  [seq_q, D] | [H, seq_q, D] | [B, H, seq_q, D]   FP16 or FP32
+//   K, V    [seq_kv, D] | [Hkv, seq_kv, D] | [B, Hkv, seq_kv, D]   FP16
+// with H a multiple of Hkv (grouped-query attention).  The extra attribute
+// `causal` (bool, default true) switches the mask off, which is what the
+// Vulkan operator computes (src/operators/vulkan/vulkan_operators.cpp:392-397).
+#include <cmath>
+#include <mutex>
+
+#include "granite/hip_backend.h"
+#include "granite/hip_compute.h"
+#include "granite/operators.h"
+#include "granite_hip.h"
+
+namespace granite {
+namespace {
+
+struct AttnDims {
+    int64_t batch = 1, heads = 1, seq = 0, dim = 0;
+};
+
+Result<AttnDims> split_dims(const Tensor& t, const char* what) {
+    AttnDims d;
+    const size_t n = t.ndim();
+    if (n < 2 || n > 4)
+        return Error(ErrorCode::InvalidShape, std::string(what) + " must have 2 to 4 dimensions");
+    d.dim = t.size(-1);
+    d.seq = t.size(-2);
+    if (n >= 3) d.heads = t.size(-3);
+    if (n == 4) d.batch = t.size(0);
+    return d;
+}
+
+class HipAttentionOp final : public IOperator {
+  public:
+    OpType type() const override { return OpType::ScaledDotProductAttention; }
+
+    Result<void> validate(const OpContext& ctx) const override {
+        if (ctx.num_inputs() < 3)
+            return Error(ErrorCode::InvalidArgument, "Attention requires 3 inputs (Q, K, V)");
+        const Tensor& Q = ctx.inputs[0];
+        const Tensor& K = ctx.inputs[1];
+        const Tensor& V = ctx.inputs[2];
+        GRANITE_TRY_ASSIGN(q, split_dims(Q, "Q"));
+        GRANITE_TRY_ASSIGN(k, split_dims(K, "K"));
+        GRANITE_TRY_ASSIGN(v, split_dims(V, "V"));
+        if (Q.ndim() != K.ndim() || K.ndim() != V.ndim())
+            return Error(ErrorCode::ShapeMismatch, "Q, K and V must have the same rank");
+        if (k.dim != q.dim || v.dim != q.dim || v.seq != k.seq || v.heads != k.heads ||
+            k.batch != q.batch || v.batch != q.batch)
+            return Error(ErrorCode::ShapeMismatch, "Q, K and V shapes do not agree");
+        if (k.heads <= 0 || q.heads % k.heads != 0)
+            return Error(ErrorCode::ShapeMismatch, "Query heads must be a multiple of KV heads");
+        if (Q.dtype() != DataType::FP16 && Q.dtype() != DataType::FP32)
+            return Error(ErrorCode::DTypeMismatch, "Q must be FP16 or FP32");
+        if (K.dtype() != DataType::FP16 || V.dtype() != DataType::FP16)
+            return Error(ErrorCode::DTypeMismatch, "K and V must be FP16 (the KV cache type)");
+        if (!Q.is_contiguous() || !K.is_contiguous() || !V.is_contiguous())
+            return Error(ErrorCode::InvalidArgument, "Q, K and V must be contiguous");
+        return {};
+    }
+
+    Result<std::vector<std::vector<int64_t>>> infer_shapes(const OpContext& ctx) const override {
+        if (ctx.num_inputs() < 1) return Error(ErrorCode::InvalidArgument, "Attention needs Q");
+        auto s = ctx.inputs[0].shape();
+        return std::vector<std::vector<int64_t>>{std::vector<int64_t>(s.begin(), s.end())};
+    }
+
+    Result<void> execute(OpContext& ctx) override {
+        GRANITE_TRY(validate(ctx));
+        if (!ctx.backend || ctx.backend->get_type() != BackendType::HIP)
+            return Error(ErrorCode::BackendNotSupported, "HipAttentionOp needs a HIP backend");
+        if (ctx.num_outputs() < 1) return Error(ErrorCode::InvalidArgument, "Attention needs an output");
+        const Tensor& Q = ctx.inputs[0];
+        const Tensor& K = ctx.inputs[1];
+        const Tensor& V = ctx.inputs[2];
+        Tensor& out = ctx.outputs[0];
+        if (out.dtype() != Q.dtype() || out.numel() != Q.numel() || !out.is_contiguous())
+            return Error(ErrorCode::ShapeMismatch, "Output must match Q in shape and dtype");
+
+        const AttnDims q = split_dims(Q, "Q").value();
+        const AttnDims k = split_dims(K, "K").value();
+        const double scale =
+            ctx.attrs.get<double>("scale", 1.0 / std::sqrt(static_cast<double>(q.dim)));
+        const int64_t start_pos = ctx.attrs.get<int64_t>("start_pos", 0);
+        const bool causal = ctx.attrs.get<bool>("causal", true);
+        if (start_pos < 0) return Error(ErrorCode::InvalidArgument, "start_pos must be >= 0");
+
+        auto base = [&](const Tensor& t) -> char* {
+            auto* p = static_cast<char*>(hip_device_pointer(ctx.backend, t.buffer()));
+            return p ? p + t.buffer_offset() : nullptr;
+        };
+        char* q_ptr = base(Q);
+        char* k_ptr = base(K);
+        char* v_ptr = base(V);
+        char* o_ptr = base(out);
+        if (!q_ptr || !k_ptr || !v_ptr || !o_ptr)
+            return Error(ErrorCode::InvalidArgument, "Tensor buffers do not belong to the HIP backend");
+
+        const int dtype = Q.dtype() == DataType::FP16 ? GRANITE_HIP_F16 : GRANITE_HIP_F32;
+        const size_t q_batch_bytes = size_t(q.heads * q.seq * q.dim) * dtype_size(Q.dtype());
+        const size_t kv_batch_bytes = size_t(k.heads * k.seq * k.dim) * sizeof(uint16_t);
+
+        HipCompute compute;  // stateless façade over the already initialised library
+        for (int64_t b = 0; b < q.batch; ++b) {
+            granite_hip_attention_args a{};
+            a.q = q_ptr + b * q_batch_bytes;
+            a.q_dtype = dtype;
+            a.q_tok_stride = q.dim;
+            a.q_head_stride = q.seq * q.dim;
+            a.out = o_ptr + b * q_batch_bytes;
+            a.out_dtype = dtype;
+            a.out_tok_stride = q.dim;
+            a.out_head_stride = q.seq * q.dim;
+            a.k_cache = k_ptr + b * kv_batch_bytes;
+            a.v_cache = v_ptr + b * kv_batch_bytes;
+            a.max_seq = static_cast<uint32_t>(k.seq);
+            a.cache_len = static_cast<uint32_t>(k.seq);
+            a.mask_mode = causal ? GRANITE_HIP_MASK_CAUSAL : GRANITE_HIP_MASK_NONE;
+            a.start_pos = static_cast<uint32_t>(start_pos);
+            a.seq_q = static_cast<uint32_t>(q.seq);
+            a.num_heads = static_cast<uint32_t>(q.heads);
+            a.num_kv_heads = static_cast<uint32_t>(k.heads);
+            a.head_dim = static_cast<uint32_t>(q.dim);
+            a.scale = static_cast<float>(scale);
+            GRANITE_TRY(compute.attention(a));
+        }
+        return {};
+    }
+};
+
+}  // namespace
+
+void register_hip_operators() {
+    static std::once_flag once;
+    std::call_once(once, [] {
+        OperatorRegistry::instance().register_op(
+            OpType::ScaledDotProductAttention, BackendType::HIP,
+            []() -> std::unique_ptr<IOperator> { return std::make_unique<HipAttentionOp>(); });
+    });
+}
+
+}  // namespace granite

@@ -1,0 +1,472 @@
+// GPU tests of the C++ host layer: HipBackend buffers, HipCompute, the
+// registered attention operator and the KV classes, checked against the CPU
+// oracle (linked as a shared library; it is the checker, never the path under
+// test).  Needs an MI355X; exits with status 77 when no usable GPU is present.
+#include <cmath>
+#include <cstring>
+#include <random>
+
+#include "check.h"
+#include "granite/hip_backend.h"
+#include "granite/hip_compute.h"
+#include "granite/kv_cache.h"
+#include "granite/operators.h"
+#include "granite_hip.h"
+
+extern "C" {
+// CPU oracle (oracle/granite_oracle.c)
+uint16_t go_fp32_to_fp16(float f);
+float go_fp16_to_fp32(uint16_t h);
+int go_kv_cache_append_f16(uint16_t* cache, const uint16_t* src, int num_kv_heads, int head_dim,
+                           int current_len, int new_len, int max_seq);
+void go_paged_kv_cache_append_f32(uint16_t* pool, const float* src, const int32_t* table,
+                                  int num_kv_heads, int head_dim, int start_pos, int new_len,
+                                  int block_size);
+void go_attention_cached(const float* q, const uint16_t* cache_k, const uint16_t* cache_v,
+                         float* context, float* lse, int batch, int seq_len, int num_heads,
+                         int num_kv_heads, int head_dim, int total_seq, int max_seq,
+                         int start_pos, float scale);
+void go_batched_paged_decode(const float* q, const uint16_t* pool_k, const uint16_t* pool_v,
+                             const int32_t* tables, const int32_t* seq_lens, float* out, float* lse,
+                             int batch, int num_heads, int num_kv_heads, int head_dim,
+                             int block_size, int max_blocks, float scale);
+int go_attention_tree(const float* q, const uint16_t* cache_k, const uint16_t* cache_v,
+                      const int32_t* table, int block_size, int max_seq, const float* k_tree,
+                      const float* v_tree, const int32_t* parent, float* context, float* lse,
+                      int batch, int num_nodes, int num_heads, int num_kv_heads, int head_dim,
+                      int cached_len, float scale);
+}
+
+using namespace granite;
+
+namespace {
+
+constexpr int D = 128;
+// Output tolerance of the attention path: max-abs 2e-3, max-rel 1e-2 (either one passes).
+bool close_enough(const std::vector<float>& got, const std::vector<float>& want, const char* what) {
+    double worst = 0;
+    size_t bad = 0;
+    for (size_t i = 0; i < want.size(); ++i) {
+        const double err = std::fabs(double(got[i]) - double(want[i]));
+        worst = std::max(worst, err);
+        if (!(err <= 2e-3 || err <= 1e-2 * std::fabs(double(want[i])))) ++bad;
+    }
+    std::printf("  %s: max abs err %.3g over %zu values\n", what, worst, want.size());
+    return bad == 0 && got.size() == want.size();
+}
+
+std::vector<float> randn(size_t n, uint32_t seed, float scale = 1.0f) {
+    std::mt19937 gen(seed);
+    std::normal_distribution<float> dist(0.0f, scale);
+    std::vector<float> v(n);
+    for (auto& x : v) x = dist(gen);
+    return v;
+}
+std::vector<uint16_t> to_half(const std::vector<float>& v) {
+    std::vector<uint16_t> h(v.size());
+    for (size_t i = 0; i < v.size(); ++i) h[i] = go_fp32_to_fp16(v[i]);
+    return h;
+}
+std::vector<float> to_float(const std::vector<uint16_t>& h) {
+    std::vector<float> v(h.size());
+    for (size_t i = 0; i < h.size(); ++i) v[i] = go_fp16_to_fp32(h[i]);
+    return v;
+}
+
+IComputeBackend* backend() {
+    static std::unique_ptr<IComputeBackend> be = [] {
+        auto b = create_backend(BackendType::HIP);
+        if (b && !b->initialize().ok()) b.reset();
+        return b;
+    }();
+    return be.get();
+}
+
+template <typename T>
+Tensor upload(std::initializer_list<int64_t> shape, DataType dt, const std::vector<T>& host) {
+    auto made = Tensor::allocate(shape, dt, backend());
+    if (!made.ok()) return Tensor{};
+    Tensor t = made.take();
+    if (!backend()->write_buffer(t.buffer(), host.data(), host.size() * sizeof(T)).ok())
+        return Tensor{};
+    return t;
+}
+template <typename T>
+std::vector<T> download(const Tensor& t) {
+    std::vector<T> host(t.size_bytes() / sizeof(T));
+    (void)backend()->wait_for_completion();
+    (void)backend()->read_buffer(t.buffer(), host.data(), t.size_bytes(), t.buffer_offset());
+    return host;
+}
+
+}  // namespace
+
+TEST_CASE(backend_buffers) {
+    IComputeBackend* be = backend();
+    REQUIRE(be != nullptr);
+    auto caps = be->get_capabilities();
+    CHECK(caps.simd_width == 64 && caps.supports_fp16 && caps.max_buffer_size > (size_t(1) << 30));
+    CHECK(caps.name != nullptr && std::strlen(caps.name) > 0);
+    CHECK(be->get_type() == BackendType::HIP && be->is_initialized());
+    CHECK(is_backend_available(BackendType::HIP) && !is_backend_available(BackendType::Metal));
+    CHECK_CODE(be->create_buffer(BufferDesc::device(0)), ErrorCode::InvalidArgument);
+
+    std::vector<uint32_t> pattern(1024);
+    for (size_t i = 0; i < pattern.size(); ++i) pattern[i] = uint32_t(i * 2654435761u);
+    for (MemoryType kind : {MemoryType::Device, MemoryType::Shared, MemoryType::Managed}) {
+        auto made = be->create_buffer({4096, kind, false});
+        REQUIRE(made.ok());
+        BufferHandle h = made.value();
+        CHECK(be->get_native_buffer(h) != nullptr);
+        CHECK_OK(be->write_buffer(h, pattern.data(), 4096));
+        std::vector<uint32_t> back(1024, 0);
+        CHECK_OK(be->read_buffer(h, back.data(), 4096));
+        CHECK(back == pattern);
+        CHECK_OK(be->read_buffer(h, back.data(), 16, 4080));
+        CHECK(back[0] == pattern[1020]);
+        CHECK_CODE(be->write_buffer(h, pattern.data(), 4096, 8), ErrorCode::BufferTooSmall);
+        CHECK_CODE(be->read_buffer(h, back.data(), 8, 4092), ErrorCode::BufferTooSmall);
+        auto mapped = be->map_buffer(h);
+        if (kind == MemoryType::Device) {
+            CHECK_CODE(mapped, ErrorCode::InvalidArgument);
+        } else {
+            REQUIRE(mapped.ok());
+            auto* p = static_cast<uint32_t*>(mapped.value());
+            CHECK(p[5] == pattern[5]);
+            p[5] = 0xdeadbeefu;  // host edit, published by unmap
+            be->unmap_buffer(h);
+            CHECK_OK(be->read_buffer(h, back.data(), 4, 20));
+            CHECK(back[0] == 0xdeadbeefu);
+        }
+        be->destroy_buffer(h);
+        CHECK(be->get_native_buffer(h) == nullptr);
+    }
+
+    auto a = be->create_buffer_from_host(pattern.data(), BufferDesc::device(4096));
+    auto b = be->create_buffer(BufferDesc::managed(4096));
+    REQUIRE(a.ok() && b.ok());
+    CHECK_OK(be->copy_buffer(a.value(), b.value(), 1024, 1024, 2048));
+    CHECK_CODE(be->copy_buffer(a.value(), b.value(), 4096, 1, 0), ErrorCode::BufferTooSmall);
+    auto fence = be->create_fence();
+    REQUIRE(fence.ok());
+    CHECK_OK(be->wait_fence(fence.value()));
+    be->destroy_fence(fence.value());
+    CHECK_CODE(be->wait_fence(fence.value()), ErrorCode::InvalidArgument);
+    std::vector<uint32_t> back(256);
+    CHECK_OK(be->read_buffer(b.value(), back.data(), 1024, 2048));
+    CHECK(std::memcmp(back.data(), pattern.data() + 256, 1024) == 0);
+    CHECK_CODE(be->create_buffer_from_host(nullptr, BufferDesc::device(16)),
+               ErrorCode::InvalidArgument);
+    CHECK_CODE(be->create_pipeline({}), ErrorCode::NotImplemented);
+    CHECK_CODE(be->dispatch(1), ErrorCode::NotImplemented);
+    CHECK_OK(be->submit());
+    be->destroy_buffer(a.value());
+    be->destroy_buffer(b.value());
+    CHECK(get_hip_compute() != nullptr && get_hip_compute()->is_initialized());
+}
+
+// The reference's attention known-answer test (tests/test_vulkan.cpp:353-482):
+// Sq=2, Skv=3, D=4, no mask, Q[i]=i+1, K^T[i]=(i+1)/2, V[i]=(i+1)/4, scale 0.5,
+// tolerance 1e-4.  All inputs are exact in binary16.  The head dimension is
+// embedded in 128 columns of zeros, which changes neither scores nor the first
+// four output columns.  Expected values: tests/golden/vulkan_attention_kat.json.
+TEST_CASE(operator_known_answer) {
+    REQUIRE(backend() != nullptr);
+    const double expected[2][4] = {
+        {2.162234681491403, 2.412234681491403, 2.662234681491403, 2.912234681491403},
+        {2.248494307269034, 2.498494307269034, 2.748494307269034, 2.998494307269034}};
+    std::vector<float> q(2 * D, 0.0f), k(3 * D, 0.0f), v(3 * D, 0.0f);
+    for (int i = 0; i < 2; ++i)
+        for (int d = 0; d < 4; ++d) q[i * D + d] = float(i * 4 + d + 1);
+    for (int d = 0; d < 4; ++d)
+        for (int t = 0; t < 3; ++t) k[t * D + d] = float(d * 3 + t + 1) * 0.5f;  // K^T is [D, T]
+    for (int t = 0; t < 3; ++t)
+        for (int d = 0; d < 4; ++d) v[t * D + d] = float(t * 4 + d + 1) * 0.25f;
+
+    initialize_operators();
+    auto op = OperatorRegistry::instance().create(OpType::ScaledDotProductAttention,
+                                                  BackendType::HIP);
+    REQUIRE(op != nullptr);
+    for (DataType qdt : {DataType::FP32, DataType::FP16}) {
+        OpContext ctx;
+        ctx.backend = backend();
+        Tensor Q = qdt == DataType::FP32 ? upload({2, D}, qdt, q) : upload({2, D}, qdt, to_half(q));
+        ctx.inputs = {Q, upload({3, D}, DataType::FP16, to_half(k)),
+                      upload({3, D}, DataType::FP16, to_half(v))};
+        auto shapes = op->infer_shapes(ctx);
+        REQUIRE(shapes.ok());
+        auto out = Tensor::allocate(shapes.value()[0], qdt, backend());
+        REQUIRE(out.ok());
+        ctx.outputs = {out.take()};
+        ctx.attrs.set("scale", 0.5);
+        ctx.attrs.set("causal", false);
+        CHECK_OK(op->validate(ctx));
+        CHECK_OK(op->execute(ctx));
+        std::vector<float> got = qdt == DataType::FP32 ? download<float>(ctx.outputs[0])
+                                                       : to_float(download<uint16_t>(ctx.outputs[0]));
+        const double tol = qdt == DataType::FP32 ? 1e-4 : 2e-3;  // fp16 output rounding
+        for (int i = 0; i < 2; ++i) {
+            for (int d = 0; d < 4; ++d) CHECK(std::fabs(got[i * D + d] - expected[i][d]) <= tol);
+            for (int d = 4; d < D; ++d) CHECK(got[i * D + d] == 0.0f);
+        }
+        for (auto& t : ctx.inputs) backend()->destroy_buffer(t.buffer());
+        backend()->destroy_buffer(ctx.outputs[0].buffer());
+    }
+}
+
+// Causal, grouped-query, chunk at start_pos > 0 through the operator, against
+// the oracle's cached attention (transformer.mm:1703-1840 restated).
+TEST_CASE(operator_causal_gqa_vs_oracle) {
+    REQUIRE(backend() != nullptr);
+    const int H = 8, Hkv = 2, Sq = 96, start = 37, Skv = start + Sq;
+    auto q = randn(size_t(H) * Sq * D, 11);                 // [H, Sq, D]
+    auto kh = to_half(randn(size_t(Hkv) * Skv * D, 12));    // [Hkv, Skv, D]
+    auto vh = to_half(randn(size_t(Hkv) * Skv * D, 13));
+    auto op = OperatorRegistry::instance().create(OpType::ScaledDotProductAttention,
+                                                  BackendType::HIP);
+    REQUIRE(op != nullptr);
+    OpContext ctx;
+    ctx.backend = backend();
+    ctx.inputs = {upload({H, Sq, D}, DataType::FP32, q), upload({Hkv, Skv, D}, DataType::FP16, kh),
+                  upload({Hkv, Skv, D}, DataType::FP16, vh)};
+    ctx.outputs = {Tensor::allocate({H, Sq, D}, DataType::FP32, backend()).take()};
+    ctx.attrs.set("start_pos", int64_t(start));
+    CHECK_OK(op->execute(ctx));  // scale defaults to 1/sqrt(D)
+    auto got = download<float>(ctx.outputs[0]);
+
+    std::vector<float> q_tok(q.size()), want_tok(q.size()), want(q.size());
+    for (int h = 0; h < H; ++h)
+        for (int s = 0; s < Sq; ++s)
+            std::memcpy(&q_tok[(size_t(s) * H + h) * D], &q[(size_t(h) * Sq + s) * D], D * 4);
+    go_attention_cached(q_tok.data(), kh.data(), vh.data(), want_tok.data(), nullptr, 1, Sq, H, Hkv,
+                        D, Skv, Skv, start, 1.0f / std::sqrt(float(D)));
+    for (int h = 0; h < H; ++h)
+        for (int s = 0; s < Sq; ++s)
+            std::memcpy(&want[(size_t(h) * Sq + s) * D], &want_tok[(size_t(s) * H + h) * D], D * 4);
+    CHECK(close_enough(got, want, "operator causal GQA"));
+    for (auto& t : ctx.inputs) backend()->destroy_buffer(t.buffer());
+    backend()->destroy_buffer(ctx.outputs[0].buffer());
+}
+
+TEST_CASE(kv_cache_append_on_device) {
+    REQUIRE(backend() != nullptr);
+    ModelConfig cfg;
+    cfg.num_layers = 2;
+    cfg.num_kv_heads = 2;
+    cfg.num_heads = 4;
+    cfg.head_dim = D;
+    const int max_seq = 64;
+    auto made = KVCache::allocate(cfg, max_seq, backend());
+    REQUIRE(made.ok());
+    KVCache cache = made.take();
+    const size_t cache_elems = size_t(cfg.num_kv_heads) * max_seq * D;
+    // the oracle appends into caches that start from the same bytes as the device's
+    std::vector<std::vector<uint16_t>> want_k, want_v;
+    for (int l = 0; l < 2; ++l) {
+        want_k.push_back(download<uint16_t>(cache.get(l).first));
+        want_v.push_back(download<uint16_t>(cache.get(l).second));
+    }
+    int len = 0;
+    uint32_t seed = 100;
+    for (int new_len : {5, 1, 26}) {
+        for (int l = 0; l < 2; ++l) {
+            auto kh = to_half(randn(size_t(2) * new_len * D, seed++));
+            auto vh = to_half(randn(size_t(2) * new_len * D, seed++));
+            Tensor nk = upload({1, 2, new_len, D}, DataType::FP16, kh);
+            Tensor nv = upload({1, 2, new_len, D}, DataType::FP16, vh);
+            CHECK_OK(cache.append(l, nk, nv));
+            CHECK(cache.seq_len() == (l == 1 ? len + new_len : len));  // advances on the last layer
+            CHECK(go_kv_cache_append_f16(want_k[l].data(), kh.data(), 2, D, len, new_len, max_seq) == 0);
+            CHECK(go_kv_cache_append_f16(want_v[l].data(), vh.data(), 2, D, len, new_len, max_seq) == 0);
+            (void)backend()->wait_for_completion();
+            backend()->destroy_buffer(nk.buffer());
+            backend()->destroy_buffer(nv.buffer());
+        }
+        len += new_len;
+    }
+    CHECK(cache.seq_len() == 32);
+    for (int l = 0; l < 2; ++l) {
+        CHECK(download<uint16_t>(cache.get(l).first) == want_k[l]);   // bit exact
+        CHECK(download<uint16_t>(cache.get(l).second) == want_v[l]);
+        CHECK(want_k[l].size() == cache_elems);
+    }
+    Tensor big = upload({1, 2, 33, D}, DataType::FP16, std::vector<uint16_t>(size_t(2) * 33 * D, 0));
+    CHECK_CODE(cache.append(0, big, big), ErrorCode::InvalidArgument);  // 32 + 33 > 64
+    CHECK(cache.seq_len() == 32);
+    cache.truncate(10);
+    CHECK(cache.seq_len() == 10);
+
+    // Attention over what the cache holds: decode one token against 10 cached rows.
+    auto q = randn(size_t(4) * D, 77);
+    Tensor Q = upload({4, 1, D}, DataType::FP32, q);
+    Tensor out = Tensor::allocate({4, 1, D}, DataType::FP32, backend()).take();
+    HipCompute* hc = get_hip_compute();
+    REQUIRE(hc != nullptr);
+    auto [ck, cv] = cache.get(1);
+    CHECK_OK(hc->multihead_attention(hip_device_pointer(backend(), Q.buffer()),
+                                     hip_device_pointer(backend(), ck.buffer()),
+                                     hip_device_pointer(backend(), cv.buffer()),
+                                     hip_device_pointer(backend(), out.buffer()), 4, 2, 1, 10, D,
+                                     0.09f, max_seq));
+    hc->sync();
+    std::vector<float> want(q.size());
+    go_attention_cached(q.data(), want_k[1].data(), want_v[1].data(), want.data(), nullptr, 1, 1, 4,
+                        2, D, 10, max_seq, 9, 0.09f);
+    CHECK(close_enough(download<float>(out), want, "decode over KVCache"));
+}
+
+TEST_CASE(paged_pool_append_and_batched_decode) {
+    REQUIRE(backend() != nullptr);
+    HipCompute* hc = get_hip_compute();
+    REQUIRE(hc != nullptr);
+    ModelConfig cfg;
+    cfg.num_layers = 1;
+    cfg.num_kv_heads = 2;
+    cfg.num_heads = 8;
+    cfg.head_dim = D;
+    const int bs = 16, batch = 3;
+    const int lens[batch] = {40, 17, 100};
+    PagedKVPool pool;
+    CHECK_OK(pool.initialize(cfg, batch, 256, bs, backend()));
+    BlockManager& mgr = pool.block_manager();
+    const size_t pool_elems = size_t(mgr.num_total_blocks()) * bs * 2 * D;
+    auto want_k = download<uint16_t>(mgr.k_cache(0));
+    auto want_v = download<uint16_t>(mgr.v_cache(0));
+    CHECK(want_k.size() == pool_elems);
+    void* k_pool = hip_device_pointer(backend(), mgr.k_cache(0).buffer());
+    void* v_pool = hip_device_pointer(backend(), mgr.v_cache(0).buffer());
+
+    // interleave the sequences' growth so that their blocks interleave too
+    int slots[batch];
+    for (int b = 0; b < batch; ++b) slots[b] = pool.acquire_slot();
+    uint32_t seed = 500;
+    int done[batch] = {0, 0, 0};
+    for (int round = 0; round < 7; ++round)
+        for (int b = 0; b < batch; ++b) {
+            const int step = std::min(lens[b] - done[b], b == 2 ? 15 : 9);
+            if (step <= 0) continue;
+            PagedKVCache& seq = pool.get_cache(slots[b]);
+            REQUIRE(seq.append_tokens(step));
+            auto nk = randn(size_t(2) * step * D, seed++);  // [Hkv, step, D] float
+            auto nv = randn(size_t(2) * step * D, seed++);
+            std::vector<int32_t> table(seq.block_table().begin(), seq.block_table().end());
+            HipBuffer* d_k = hc->create_buffer(nk.size() * 4);
+            HipBuffer* d_v = hc->create_buffer(nv.size() * 4);
+            HipBuffer* d_t = hc->create_buffer(table.size() * 4);
+            REQUIRE(d_k && d_v && d_t);
+            CHECK_OK(hc->upload(d_k, nk.data(), nk.size() * 4));
+            CHECK_OK(hc->upload(d_v, nv.data(), nv.size() * 4));
+            CHECK_OK(hc->upload(d_t, table.data(), table.size() * 4));
+            CHECK_OK(hc->paged_kv_cache_append(d_k, d_v, k_pool, v_pool, d_t, 2, D, done[b], step, bs));
+            hc->sync();
+            go_paged_kv_cache_append_f32(want_k.data(), nk.data(), table.data(), 2, D, done[b], step, bs);
+            go_paged_kv_cache_append_f32(want_v.data(), nv.data(), table.data(), 2, D, done[b], step, bs);
+            hc->release_buffer(d_k);
+            hc->release_buffer(d_v);
+            hc->release_buffer(d_t);
+            done[b] += step;
+        }
+    for (int b = 0; b < batch; ++b) CHECK(pool.get_cache(slots[b]).seq_len() == lens[b]);
+    CHECK(download<uint16_t>(mgr.k_cache(0)) == want_k);  // bit exact
+    CHECK(download<uint16_t>(mgr.v_cache(0)) == want_v);
+
+    const int max_blocks = 8;
+    std::vector<int32_t> tables(size_t(batch) * max_blocks, 0), seq_lens(lens, lens + batch);
+    for (int b = 0; b < batch; ++b) {
+        const auto& t = pool.get_cache(slots[b]).block_table();
+        std::copy(t.begin(), t.end(), tables.begin() + size_t(b) * max_blocks);
+    }
+    auto q = randn(size_t(batch) * 8 * D, 900);
+    HipBuffer* d_q = hc->create_buffer(q.size() * 4);
+    HipBuffer* d_o = hc->create_buffer(q.size() * 4);
+    HipBuffer* d_t = hc->create_buffer(tables.size() * 4);
+    HipBuffer* d_l = hc->create_buffer(seq_lens.size() * 4);
+    REQUIRE(d_q && d_o && d_t && d_l);
+    CHECK_OK(hc->upload(d_q, q.data(), q.size() * 4));
+    CHECK_OK(hc->upload(d_t, tables.data(), tables.size() * 4));
+    CHECK_OK(hc->upload(d_l, seq_lens.data(), seq_lens.size() * 4));
+    const float scale = 1.0f / std::sqrt(float(D));
+    CHECK_OK(hc->batched_paged_attention_decode(d_q, k_pool, v_pool, d_t, d_l, d_o, batch, 8, 2, D,
+                                                bs, max_blocks, scale));
+    std::vector<float> got(q.size()), want(q.size());
+    CHECK_OK(hc->download(got.data(), d_o, got.size() * 4));
+    go_batched_paged_decode(q.data(), want_k.data(), want_v.data(), tables.data(), seq_lens.data(),
+                            want.data(), nullptr, batch, 8, 2, D, bs, max_blocks, scale);
+    CHECK(close_enough(got, want, "batched paged decode"));
+
+    // single-sequence entry point on the longest sequence
+    std::vector<float> got1(size_t(8) * D), want1(want.begin() + size_t(2) * 8 * D, want.end());
+    CHECK_OK(hc->paged_attention_decode(static_cast<char*>(d_q) + size_t(2) * 8 * D * 4, k_pool, v_pool,
+                                        static_cast<char*>(d_t) + size_t(2) * max_blocks * 4, d_o, 8, 2,
+                                        lens[2], D, bs, scale));
+    CHECK_OK(hc->download(got1.data(), d_o, got1.size() * 4));
+    CHECK(close_enough(got1, want1, "paged decode, one sequence"));
+    for (HipBuffer* p : {d_q, d_o, d_t, d_l}) hc->release_buffer(p);
+    for (int b = 0; b < batch; ++b) pool.release_slot(slots[b]);
+    CHECK(pool.num_free_blocks() == mgr.num_total_blocks());
+}
+
+TEST_CASE(speculation_tree_attention) {
+    REQUIRE(backend() != nullptr);
+    HipCompute* hc = get_hip_compute();
+    REQUIRE(hc != nullptr);
+    SpeculationTree tree;
+    tree.add_node(1, -1);
+    std::mt19937 gen(4242);
+    for (int i = 1; i < 23; ++i) tree.add_node(i + 1, int(gen() % uint32_t(i)));
+    const std::vector<int> parents_int = tree.get_parent_indices();
+    std::vector<int32_t> parents(parents_int.begin(), parents_int.end());
+    const int N = int(tree.size()), H = 4, Hkv = 2, cache_len = 75;
+    auto q = randn(size_t(H) * N * D, 31);                       // [H, N, D]
+    auto ck = to_half(randn(size_t(Hkv) * cache_len * D, 32));   // [Hkv, cache_len, D]
+    auto cv = to_half(randn(size_t(Hkv) * cache_len * D, 33));
+    auto tk = to_half(randn(size_t(Hkv) * N * D, 34));           // [Hkv, N, D]
+    auto tv = to_half(randn(size_t(Hkv) * N * D, 35));
+    const float scale = 0.1f;
+
+    auto dev = [&](const void* p, size_t bytes) {
+        HipBuffer* d = hc->create_buffer(bytes);
+        if (d) (void)hc->upload(d, p, bytes);
+        return d;
+    };
+    HipBuffer* d_q = dev(q.data(), q.size() * 4);
+    HipBuffer* d_ck = dev(ck.data(), ck.size() * 2);
+    HipBuffer* d_cv = dev(cv.data(), cv.size() * 2);
+    HipBuffer* d_tk = dev(tk.data(), tk.size() * 2);
+    HipBuffer* d_tv = dev(tv.data(), tv.size() * 2);
+    HipBuffer* d_p = dev(parents.data(), parents.size() * 4);
+    HipBuffer* d_o = hc->create_buffer(q.size() * 4);
+    REQUIRE(d_q && d_ck && d_cv && d_tk && d_tv && d_p && d_o);
+    CHECK_OK(hc->attention_tree(d_q, d_ck, d_cv, d_tk, d_tv, d_p, d_o, H, Hkv, N, cache_len, D, scale));
+    std::vector<float> got(q.size());
+    CHECK_OK(hc->download(got.data(), d_o, got.size() * 4));
+
+    // oracle layouts: q [N, H, D], tree K/V [N, Hkv, D] floats, output [N, H*D]
+    std::vector<float> q_tok(q.size()), tkf(tk.size()), tvf(tv.size()), want_tok(q.size()),
+        want(q.size());
+    auto tk32 = to_float(tk), tv32 = to_float(tv);
+    for (int h = 0; h < H; ++h)
+        for (int n = 0; n < N; ++n)
+            std::memcpy(&q_tok[(size_t(n) * H + h) * D], &q[(size_t(h) * N + n) * D], D * 4);
+    for (int h = 0; h < Hkv; ++h)
+        for (int n = 0; n < N; ++n) {
+            std::memcpy(&tkf[(size_t(n) * Hkv + h) * D], &tk32[(size_t(h) * N + n) * D], D * 4);
+            std::memcpy(&tvf[(size_t(n) * Hkv + h) * D], &tv32[(size_t(h) * N + n) * D], D * 4);
+        }
+    CHECK(go_attention_tree(q_tok.data(), ck.data(), cv.data(), nullptr, 0, cache_len, tkf.data(),
+                            tvf.data(), parents.data(), want_tok.data(), nullptr, 1, N, H, Hkv, D,
+                            cache_len, scale) == 0);
+    for (int h = 0; h < H; ++h)
+        for (int n = 0; n < N; ++n)
+            std::memcpy(&want[(size_t(h) * N + n) * D], &want_tok[(size_t(n) * H + h) * D], D * 4);
+    CHECK(close_enough(got, want, "tree attention over SpeculationTree parents"));
+    for (HipBuffer* p : {d_q, d_ck, d_cv, d_tk, d_tv, d_p, d_o}) hc->release_buffer(p);
+}
+
+int main(int argc, char** argv) {
+    if (!backend()) {
+        std::printf("no usable gfx950 GPU: skipping\n");
+        return 77;
+    }
+    return hosttest::run_all(argc, argv);
+}
