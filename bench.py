@@ -41,6 +41,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (see profiles/); None until measured.
+CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
+
 MEASURED_TRAFFIC = {
     "paged_decode": None,
     "prefill": None,
@@ -138,14 +140,16 @@ def bench_paged_decode(gpu, steps, warmup, cpu):
         import oracle_bind
         oracle = oracle_bind.load()
         q32 = c.q.astype(np.float32)
-        t0 = time.perf_counter()
-        want, want_lse = oracle.batched_paged_decode(q32, c.k_pool, c.v_pool, c.block_tables, c.seq_lens,
-                                                     c.block_size, c.scale)
-        cpu_s = time.perf_counter() - t0
+        passes, t0 = 0, time.perf_counter()
+        while passes == 0 or time.perf_counter() - t0 < CPU_SAMPLE_SECONDS:
+            want, want_lse = oracle.batched_paged_decode(q32, c.k_pool, c.v_pool, c.block_tables, c.seq_lens,
+                                                         c.block_size, c.scale)
+            passes += 1
+        cpu_s = (time.perf_counter() - t0) / passes
         res["cpu_baseline"] = {"value": round(nbytes / cpu_s / 1e9, 3), "unit": "GB/s",
                                "cores": oracle.lib.go_get_num_threads(), "kind": "port",
-                               "seconds": round(cpu_s, 2),
-                               "sample": "the whole workload (all 64 sequences), one pass"}
+                               "seconds": round(cpu_s * passes, 2),
+                               "sample": f"the whole workload (all 64 sequences), mean of {passes} passes"}
         res["parity"] = {"max_abs_err": max_err(out.read(np.float32, (B, hq, 128)), want),
                          "max_lse_err": max_err(lse.read(np.float32, (B, hq)), want_lse)}
     return res
@@ -178,7 +182,9 @@ def bench_prefill(gpu, steps, warmup, cpu):
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()
-        rows = list(range(0, S, 16))  # every 16th query row, all heads
+        # every 16th query row first (the parity sample), then the rows between
+        # them until the time box is used up
+        rows = list(range(0, S, 16)) + list(range(8, S, 16)) + list(range(4, S, 8)) + list(range(2, S, 4))
         k = np.ascontiguousarray(np.transpose(c.k_cache, (1, 0, 2))).astype(np.float32)
         v = np.ascontiguousarray(np.transpose(c.v_cache, (1, 0, 2))).astype(np.float32)
         got = out.read(np.float16, (S, hq, 128)).astype(np.float32)
@@ -186,18 +192,22 @@ def bench_prefill(gpu, steps, warmup, cpu):
         t0 = time.perf_counter()
         err = lerr = 0.0
         sample_flops = 0
+        done = 0
         for r in rows:
+            if done >= S // 16 and time.perf_counter() - t0 > CPU_SAMPLE_SECONDS:
+                break
             want, wl = oracle.attention_core(c.q[None, r:r + 1].astype(np.float32), k[:r + 1], v[:r + 1], r,
                                              c.scale)
             sample_flops += 4 * hq * 128 * (r + 1)
             err = max(err, max_err(got[r], want[0, 0]))
             lerr = max(lerr, max_err(got_lse[:, r], wl[0, :, 0]))
+            done += 1
         cpu_s = time.perf_counter() - t0
         res["cpu_baseline"] = {"value": round(sample_flops / cpu_s / 1e12, 5), "unit": "TFLOP/s",
                                "cores": oracle.lib.go_get_num_threads(), "kind": "port",
                                "seconds": round(cpu_s, 2),
-                               "sample": f"every 16th query row ({len(rows)} rows x {hq} heads), "
-                                         "attention core only (no cache gather)"}
+                               "sample": f"{done} of {S} query rows (every 16th, then the rows between) "
+                                         f"x {hq} heads, attention core only (no cache gather)"}
         res["parity"] = {"max_abs_err": err, "max_lse_err": lerr}
     return res
 
@@ -240,11 +250,15 @@ def bench_chunked_prefill(gpu, steps, warmup, cpu):
         k32, v32 = k_all.astype(np.float32), v_all.astype(np.float32)
         got = out.read(np.float16, (chunk, hq, 128)).astype(np.float32)
         got_lse = lse.read(np.float32, (hq, chunk))
-        rows = [0, 73, 146, 219, 292, 365, 438, 511]
+        rows = [0, 73, 146, 219, 292, 365, 438, 511] + list(range(5, chunk, 11))
         t0 = time.perf_counter()
         err = lerr = 0.0
         sample_flops = 0
+        done = 0
         for r in rows:
+            if done >= 8 and time.perf_counter() - t0 > CPU_SAMPLE_SECONDS:
+                break
+            done += 1
             want, wl = oracle.attention_core(c.q[None, r:r + 1].astype(np.float32), k32[:prefix + r + 1],
                                              v32[:prefix + r + 1], prefix + r, c.scale)
             sample_flops += 4 * hq * 128 * (prefix + r + 1)
@@ -254,7 +268,7 @@ def bench_chunked_prefill(gpu, steps, warmup, cpu):
         res["cpu_baseline"] = {"value": round(sample_flops / cpu_s / 1e12, 5), "unit": "TFLOP/s",
                                "cores": oracle.lib.go_get_num_threads(), "kind": "port",
                                "seconds": round(cpu_s, 2),
-                               "sample": f"{len(rows)} of 512 query rows x {hq} heads, attention core only"}
+                               "sample": f"{done} of 512 query rows x {hq} heads, attention core only"}
         res["parity"] = {"max_abs_err": err, "max_lse_err": lerr}
     return res
 
@@ -291,13 +305,15 @@ def bench_tree(gpu, steps, warmup, cpu):
         q = np.transpose(c.q, (1, 0, 2))[None]
         kt = np.transpose(c.k_tree, (1, 0, 2))[None].astype(np.float32)
         vt = np.transpose(c.v_tree, (1, 0, 2))[None].astype(np.float32)
-        t0 = time.perf_counter()
-        ctx, wl = oracle.attention_tree(q, c.k_pool, c.v_pool, kt, vt, c.parents, c.prefix_len, c.scale,
-                                        table=c.block_table, block_size=c.block_size)
-        cpu_s = time.perf_counter() - t0
+        passes, t0 = 0, time.perf_counter()
+        while passes == 0 or time.perf_counter() - t0 < CPU_SAMPLE_SECONDS / 2:
+            ctx, wl = oracle.attention_tree(q, c.k_pool, c.v_pool, kt, vt, c.parents, c.prefix_len, c.scale,
+                                            table=c.block_table, block_size=c.block_size)
+            passes += 1
+        cpu_s = (time.perf_counter() - t0) / passes
         res["cpu_baseline"] = {"value": round(cpu_s * 1e6, 1), "unit": "us",
                                "cores": oracle.lib.go_get_num_threads(), "kind": "port",
-                               "sample": "the whole workload, one pass (incl. the prefix gather)"}
+                               "sample": f"the whole workload, mean of {passes} passes (incl. the prefix gather)"}
         res["parity"] = {"max_abs_err": max_err(out.read(np.float32, (hq, n, 128)), np.transpose(ctx[0], (1, 0, 2))),
                          "max_lse_err": max_err(lse.read(np.float32, (hq, n)), wl[0])}
     return res
@@ -326,11 +342,11 @@ def bench_decode_contiguous(gpu, steps, warmup, cpu):
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()
-        reps = 20
-        t0 = time.perf_counter()
-        for _ in range(reps):
+        reps, t0 = 0, time.perf_counter()
+        while reps < 20 or time.perf_counter() - t0 < CPU_SAMPLE_SECONDS / 2:
             want, wl = oracle.attention_cached(c.q[None, None], c.k_cache, c.v_cache, c.seq_kv, c.seq_kv - 1,
                                                c.scale)
+            reps += 1
         cpu_s = (time.perf_counter() - t0) / reps
         res["cpu_baseline"] = {"value": round(cpu_s * 1e6, 1), "unit": "us",
                                "cores": oracle.lib.go_get_num_threads(), "kind": "port",
@@ -340,6 +356,33 @@ def bench_decode_contiguous(gpu, steps, warmup, cpu):
     return res
 
 
+def bench_copy_calibration(gpu, steps, warmup, cpu):
+    """A plain copy of known size: the block-table gather with an identity
+    table moves 2 x 128 MiB in and 2 x 128 MiB out.  Run under
+    `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` it gives the factor between a
+    counter's reading and real HBM bytes.  Not part of `--workload all`."""
+    from granite_amd import DeviceBuffer
+    hkv, d, bs, n_tok = 8, 128, 16, 65536
+    rng = np.random.default_rng(7)
+    pool = rng.integers(0, 1 << 16, size=(n_tok, hkv, d), dtype=np.uint16)
+    table = np.arange(n_tok // bs, dtype=np.int32)
+    dk, dv, dt = (DeviceBuffer.from_numpy(x) for x in (pool, pool[::-1].copy(), table))
+    ok = DeviceBuffer.from_numpy(np.zeros((hkv, n_tok, d), np.uint16))
+    ov = DeviceBuffer.from_numpy(np.zeros((hkv, n_tok, d), np.uint16))
+
+    def step():
+        gpu.paged_kv_gather(ok, ov, dk, dv, dt, hkv, d, n_tok, bs, n_tok)
+
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    moved = 2 * pool.nbytes
+    got = ok.read(np.uint16, (hkv, n_tok, d))
+    return {"workload": "copy_calibration_gather_identity_65536tok_hkv8_d128", "metric": "copy_GBps",
+            "unit": "GB/s", "value": round(2 * moved / (ms * 1e-3) / 1e9, 1), "ms_per_step": round(ms, 4),
+            "wall_ms_per_step": round(wall_ms, 4), "bytes_read": moved, "bytes_written": moved,
+            "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+            "parity": {"bit_exact": bool(np.array_equal(got, np.transpose(pool, (1, 0, 2))))}}
+
+
 WORKLOADS = {
     "paged_decode": bench_paged_decode,
     "prefill": bench_prefill,
@@ -347,6 +390,7 @@ WORKLOADS = {
     "tree": bench_tree,
     "decode_contiguous": bench_decode_contiguous,
 }
+EXTRA_WORKLOADS = {"copy_calibration": bench_copy_calibration}
 
 
 def main() -> int:
@@ -354,7 +398,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS])
+    ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS, *EXTRA_WORKLOADS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -371,7 +415,8 @@ def main() -> int:
     results = {}
     for name in names:
         t0 = time.perf_counter()
-        results[name] = WORKLOADS[name](gpu, args.steps, args.warmup, not args.no_cpu)
+        fn = WORKLOADS.get(name) or EXTRA_WORKLOADS[name]
+        results[name] = fn(gpu, args.steps, args.warmup, not args.no_cpu)
         log(f"[{name}] {results[name]['value']} {results[name]['unit']} "
             f"({results[name]['ms_per_step']} ms/step; {time.perf_counter() - t0:.1f}s total)")
 
