@@ -1,5 +1,5 @@
 // Operator plug-in surface (reference: include/granite/operators.h:20-290,
-// src/operators/operator_registry.cpp:10-54): OpType, Attributes, OpContext,
+// src/core/operator_registry.cpp:10-54): OpType, Attributes, OpContext,
 // IOperator and the (op, backend) -> factory registry.  The HIP backend
 // registers ScaledDotProductAttention through register_hip_operators(), the
 // same hook shape as register_metal_operators().

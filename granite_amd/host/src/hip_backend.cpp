@@ -14,6 +14,7 @@
 #include <unordered_map>
 
 #include "granite/hip_compute.h"
+#include "granite/operators.h"
 #include "granite_hip.h"
 
 namespace granite {
@@ -272,6 +273,7 @@ void* hip_device_pointer(IComputeBackend* backend, BufferHandle handle) {
 // The factory of this library knows one backend (src/core/backend_factory.cpp:12-40
 // is where the reference lists its own).
 std::unique_ptr<IComputeBackend> create_backend(BackendType type) {
+    initialize_operators();  // as the reference does on first backend creation (:36-37)
     return type == BackendType::HIP ? create_hip_backend() : nullptr;
 }
 std::unique_ptr<IComputeBackend> create_default_backend() { return create_hip_backend(); }
