@@ -353,7 +353,8 @@ int launch_decode(const granite_hip_decode_args& a) {
     if (use_stream_kernel()) {
         const uint64_t units = uint64_t(p.batch) * ((p.max_tokens + kTile - 1) / kTile) *
                                p.num_kv_heads * p.q_groups;
-        if (units < (1ull << 31)) return launch_decode_stream(p, qf32, rows);
+        if (units < (1ull << 31) && decode_stream_supports(p.batch))
+            return launch_decode_stream(p, qf32, rows);
     }
 
     const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;

@@ -13,7 +13,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
 struct DecodeParams {
-    uint32_t* plan;  // stream kernel: [per, total, pad, pad, prefix[batch + 1]]
+    uint32_t* plan;  // stream kernel, for its merge: [per, total, pad, pad, prefix[batch + 1]]
     const void* q;
     const uint16_t* k;
     const uint16_t* v;
@@ -29,6 +29,7 @@ struct DecodeParams {
     int64_t tok_stride, head_stride;
     uint32_t max_tokens;  // bound on any sequence length
     uint32_t chunk_tokens, max_chunks;
+    uint32_t workers, min_per;  // stream kernel: waves in the grid, smallest share of a wave
     float scale_log2;
 };
 
@@ -68,6 +69,10 @@ __device__ __forceinline__ uint32_t lane_read(uint32_t v, uint32_t src_lane) {
 
 constexpr uint32_t kPlanHeader = 4;  // words in front of prefix[]
 
+// The stream kernel keeps the prefix sums and the sequence lengths in LDS
+// (60 KiB at most); larger batches go through the chunk kernel.
+constexpr uint32_t kStreamMaxPrefix = 7680;
+bool decode_stream_supports(uint32_t batch);
 int launch_decode_stream(DecodeParams p, bool q_f32, int rows);
 
 }  // namespace ghip

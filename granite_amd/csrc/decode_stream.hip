@@ -11,6 +11,12 @@
 // the partials of a (sequence, head), whose positions follow from the same
 // arithmetic.
 //
+// There is no separate planning launch: every workgroup scans the sequence
+// lengths into tile counts and their prefix sums itself, in LDS (a few hundred
+// nanoseconds for a batch of 64), and looks everything up there afterwards, so
+// that none of the bookkeeping ever waits on global memory.  Workgroup 0 also
+// stores the prefix sums and the per-wave share for the merge kernel.
+//
 // Inside a wave the pipeline is three tiles deep: the block-table rows of tile
 // i+2 and the K/V rows of tile i+1 are in flight while tile i goes through the
 // MFMAs (two register buffers, no LDS, no barriers).  The per-tile math and
@@ -40,7 +46,9 @@ __device__ __forceinline__ uint32_t seq_len_of(const DecodeParams& p, uint32_t b
 // Next tile in (sequence, head, tile) order; skips empty sequences.  `more`
 // false leaves the cursor where it is (the caller re-reads the last tile
 // instead of running off the end, so no load ever sits inside a branch).
-__device__ __forceinline__ void advance(const DecodeParams& p, Cursor& c, bool more) {
+// `lens` holds the token count of every sequence, in LDS.
+__device__ __forceinline__ void advance(const DecodeParams& p, const uint32_t* lens, Cursor& c,
+                                        bool more) {
     if (!more) return;
     if (++c.t < c.nt) return;
     c.t = 0;
@@ -48,7 +56,7 @@ __device__ __forceinline__ void advance(const DecodeParams& p, Cursor& c, bool m
     c.vh = 0;
     do {
         ++c.b;
-        c.len = c.b < p.batch ? seq_len_of(p, c.b) : kTile;
+        c.len = c.b < p.batch ? uint32_t(__builtin_amdgcn_readfirstlane(int(lens[c.b]))) : kTile;
         c.nt = (c.len + kTile - 1) / kTile;
     } while (c.nt == 0 && c.b < p.batch);
     if (c.b >= p.batch) c.b = p.batch - 1;  // never dereferenced past the end
@@ -69,11 +77,61 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
     const uint32_t worker =
         uint32_t(__builtin_amdgcn_readfirstlane(int(blockIdx.x * kWavesPerWG + wave)));
 
-    // ---- this wave's range of the flat tile list
-    const uint32_t* prefix = p.plan + kPlanHeader;  // prefix[b] = tiles of sequences < b
-    const uint32_t per = p.plan[0];
-    const uint32_t total = p.plan[1];
+    // ---- tile counts and their prefix sums, in LDS
+    extern __shared__ uint32_t s_dyn[];
+    uint32_t* s_prefix = s_dyn;             // [batch + 1]: tiles of the sequences before b
+    uint32_t* s_len = s_dyn + p.batch + 1;  // [batch]: tokens of sequence b
+    __shared__ uint32_t s_wave_sum[kWavesPerWG];
     const uint32_t vheads = p.num_kv_heads * p.q_groups;
+    uint32_t tiles_total;
+    {
+        // every thread sums a run of consecutive sequences, the runs are scanned
+        const uint32_t run = (p.batch + blockDim.x - 1) / blockDim.x;
+        const uint32_t b0 = threadIdx.x * run;
+        uint32_t mine = 0;
+        for (uint32_t b = b0; b < min(b0 + run, p.batch); b++) {
+            const uint32_t len = seq_len_of(p, b);
+            s_len[b] = len;
+            mine += (len + kTile - 1) / kTile;
+        }
+        uint32_t incl = mine;  // inclusive scan inside the wave
+#pragma unroll
+        for (uint32_t off = 1; off < kWave; off <<= 1) {
+            const uint32_t up = lane_read(incl, lane >= off ? lane - off : lane);
+            if (lane >= off) incl += up;
+        }
+        if (lane == kWave - 1) s_wave_sum[wave] = incl;
+        __syncthreads();
+        uint32_t before = 0, all = 0;
+#pragma unroll
+        for (uint32_t w = 0; w < kWavesPerWG; w++) {
+            const uint32_t v = s_wave_sum[w];
+            if (w < wave) before += v;
+            all += v;
+        }
+        uint32_t at = before + incl - mine;
+        for (uint32_t b = b0; b < min(b0 + run, p.batch); b++) {
+            s_prefix[b] = at;
+            at += (s_len[b] + kTile - 1) / kTile;
+        }
+        tiles_total = uint32_t(__builtin_amdgcn_readfirstlane(int(all)));
+        if (threadIdx.x == 0) s_prefix[p.batch] = tiles_total;
+        __syncthreads();
+    }
+    const uint32_t total = tiles_total * vheads;
+    const uint32_t per = max((total + p.workers - 1) / p.workers, p.min_per);
+    if (blockIdx.x == 0) {  // for the merge kernel
+        for (uint32_t i = threadIdx.x; i <= p.batch; i += blockDim.x) p.plan[kPlanHeader + i] = s_prefix[i];
+        if (threadIdx.x == 0) {
+            p.plan[0] = per;
+            p.plan[1] = total;
+        }
+    }
+    auto prefix_u = [&](uint32_t i) -> uint32_t {  // wave-uniform index: stays in a scalar register
+        return uint32_t(__builtin_amdgcn_readfirstlane(int(s_prefix[i])));
+    };
+
+    // ---- this wave's range of the flat tile list
     const uint32_t u0 = worker * per;
     if (u0 >= total) return;
     const uint32_t n_units = min(per, total - u0);
@@ -84,12 +142,12 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
         uint32_t lo = 0, hi = p.batch;  // invariant: prefix[lo]*vheads <= u0 < prefix[hi]*vheads
         while (hi - lo > 1) {
             const uint32_t mid = (lo + hi) >> 1;
-            if (prefix[mid] * vheads <= u0) lo = mid; else hi = mid;
+            if (prefix_u(mid) * vheads <= u0) lo = mid; else hi = mid;
         }
         first.b = lo;
-        first.nt = prefix[lo + 1] - prefix[lo];
-        first.len = seq_len_of(p, lo);
-        const uint32_t in_seq = u0 - prefix[lo] * vheads;
+        first.nt = prefix_u(lo + 1) - prefix_u(lo);
+        first.len = uint32_t(__builtin_amdgcn_readfirstlane(int(s_len[lo])));
+        const uint32_t in_seq = u0 - prefix_u(lo) * vheads;
         first.vh = in_seq / first.nt;
         first.t = in_seq - first.vh * first.nt;
     }
@@ -224,7 +282,7 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
         const uint32_t q_in_group = qg * 16 + n;
         if (q_in_group < p.group) {
             // slot = this worker's rank among the workers that touch (b, vh)
-            const uint32_t u_start = (prefix[c.b] * vheads) + c.vh * c.nt;
+            const uint32_t u_start = prefix_u(c.b) * vheads + c.vh * c.nt;
             const uint32_t slot = worker - u_start / per;
             const size_t head = size_t(c.b) * p.num_heads + kvh * p.group + q_in_group;
             const size_t at = head * p.max_chunks + slot;
@@ -257,26 +315,26 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
     TileRegs ra, rb;
 
     uint32_t rows_a = rows_of(cr);
-    advance(p, cr, 1 < n_units);
+    advance(p, s_len, cr, 1 < n_units);
     uint32_t rows_b = rows_of(cr);
-    advance(p, cr, 2 < n_units);
+    advance(p, s_len, cr, 2 < n_units);
     issue(ra, rows_a, cl);
-    advance(p, cl, 1 < n_units);
+    advance(p, s_len, cl, 1 < n_units);
     load_q(cc);
 
     for (uint32_t i = 0; i < n_units; i += 2) {
         // tile i+1 (or tile i again at the very end) into buffer B
         issue(rb, rows_b, cl);
-        advance(p, cl, i + 2 < n_units);
+        advance(p, s_len, cl, i + 2 < n_units);
         rows_a = rows_of(cr);
-        advance(p, cr, i + 3 < n_units);
+        advance(p, s_len, cr, i + 3 < n_units);
 
         compute(ra, cc);
         {
             const bool last = i + 1 >= n_units;
             const bool seg_end = last || cc.t + 1 == cc.nt;
             const Cursor done = cc;
-            advance(p, cc, !last);
+            advance(p, s_len, cc, !last);
             if (seg_end) {
                 flush(done);
                 if (!last) load_q(cc);
@@ -285,59 +343,21 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
         }
 
         issue(ra, rows_a, cl);
-        advance(p, cl, i + 3 < n_units);
+        advance(p, s_len, cl, i + 3 < n_units);
         rows_b = rows_of(cr);
-        advance(p, cr, i + 4 < n_units);
+        advance(p, s_len, cr, i + 4 < n_units);
 
         compute(rb, cc);
         {
             const bool last = i + 2 >= n_units;
             const bool seg_end = last || cc.t + 1 == cc.nt;
             const Cursor done = cc;
-            advance(p, cc, !last);
+            advance(p, s_len, cc, !last);
             if (seg_end) {
                 flush(done);
                 if (!last) load_q(cc);
             }
         }
-    }
-}
-
-// Tiles per sequence, their exclusive prefix sums and the per-wave share of the
-// flat tile list.  One workgroup; the batch is walked in strides of 256.
-__global__ void __launch_bounds__(256) decode_plan_kernel(DecodeParams p, uint32_t workers,
-                                                          uint32_t min_per) {
-    __shared__ uint32_t s_sum[256];
-    __shared__ uint32_t s_base;
-    uint32_t* plan = p.plan;
-    uint32_t* prefix = plan + kPlanHeader;
-    if (threadIdx.x == 0) s_base = 0;
-    __syncthreads();
-    for (uint32_t b0 = 0; b0 < p.batch; b0 += 256) {
-        const uint32_t b = b0 + threadIdx.x;
-        const uint32_t nt = b < p.batch ? (seq_len_of(p, b) + kTile - 1) / kTile : 0;
-        s_sum[threadIdx.x] = nt;
-        __syncthreads();
-        for (uint32_t off = 1; off < 256; off <<= 1) {  // inclusive scan
-            const uint32_t v = threadIdx.x >= off ? s_sum[threadIdx.x - off] : 0;
-            __syncthreads();
-            s_sum[threadIdx.x] += v;
-            __syncthreads();
-        }
-        const uint32_t base = s_base;
-        if (b < p.batch) prefix[b] = base + s_sum[threadIdx.x] - nt;
-        __syncthreads();
-        if (threadIdx.x == 255) s_base = base + s_sum[255];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        const uint32_t tiles = s_base;
-        prefix[p.batch] = tiles;
-        const uint32_t total = tiles * p.num_kv_heads * p.q_groups;
-        uint32_t per = (total + workers - 1) / workers;
-        per = max(per, min_per);
-        plan[0] = per;
-        plan[1] = total;
     }
 }
 
@@ -374,7 +394,10 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
 
 }  // namespace
 
+bool decode_stream_supports(uint32_t batch) { return batch + 1 <= kStreamMaxPrefix; }
+
 int launch_decode_stream(DecodeParams p, bool q_f32, int rows) {
+    if (!decode_stream_supports(p.batch)) return GRANITE_HIP_EINVAL;
     // Workers: one wave per SIMD on every CU.
     const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
     const uint32_t wgs = cus;
@@ -396,19 +419,17 @@ int launch_decode_stream(DecodeParams p, bool q_f32, int rows) {
     p.part_o = reinterpret_cast<float*>(ws + plan_bytes);
     p.part_ml = p.part_o + slots * kHeadDim;
 
+    p.workers = workers;
+    p.min_per = min_per;
+    const size_t lds_bytes = (2 * size_t(p.batch) + 1) * sizeof(uint32_t);
+
     hipStream_t st = ctx().stream;
-    {
-        KernelTimerScope timer("decode_plan");
-        decode_plan_kernel<<<dim3(1), dim3(256), 0, st>>>(p, workers, min_per);
-    }
-    rc = launch_status();
-    if (rc != GRANITE_HIP_OK) return rc;
     {
         KernelTimerScope timer("decode_stream");
         dim3 grid(wgs), block(kWavesPerWG * kWave);
 #define GHIP_STREAM_CASE(QF32, ROWS)                               \
     if (q_f32 == QF32 && rows == ROWS)                             \
-        decode_stream_kernel<QF32, ROWS><<<grid, block, 0, st>>>(p);
+        decode_stream_kernel<QF32, ROWS><<<grid, block, lds_bytes, st>>>(p);
         GHIP_STREAM_CASE(true, kRowsContiguous)
         GHIP_STREAM_CASE(true, kRowsPagedPow2)
         GHIP_STREAM_CASE(true, kRowsPagedAny)

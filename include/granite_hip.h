@@ -114,8 +114,8 @@ int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
 /* Per-kernel GPU time, bucketed by kernel name (MetalCompute::enable_kernel_timing,
  * reset_kernel_timing, get_kernel_timing_stats; include/granite/metal_compute.h:51-59).
  * While enabled every launch is bracketed by two events on the launch stream.
- * Names: "kv_append", "kv_gather", "decode_splitk", "decode_merge",
- * "attention_tiles", "tree_mask".  granite_hip_kernel_timing_names() writes the
+ * Names: "kv_append", "kv_gather", "decode_stream" or "decode_splitk",
+ * "decode_merge", "attention_tiles", "attention_merge", "tree_mask".  granite_hip_kernel_timing_names() writes the
  * names seen so far, comma separated. */
 int granite_hip_enable_kernel_timing(int enable);
 int granite_hip_reset_kernel_timing(void);
