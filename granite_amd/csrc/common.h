@@ -87,6 +87,8 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
 
 // Granite's truncating float->half (src/llm/math_ops.cpp:45-54), bit for bit.
 __device__ __forceinline__ uint16_t f32_to_f16_truncate(float f) {

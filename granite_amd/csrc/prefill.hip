@@ -21,19 +21,28 @@
 //
 // Computing the transposed products makes the softmax output of the first
 // MFMA land exactly in the B-operand layout of the second once the keys of
-// each 16-key group are stored in LDS in the order 8g + 4a + b for key
-// 8a + 4g + b (a, g in {0,1}, b in 0..3).
+// each 16-key step are taken in the order described next.
+//
+// With the keys of a tile in their natural order the lane that owns S^T rows
+// (keys) 8a + 4g + b needs, as B operand of the second MFMA, k-index
+// 8g + 4a' + b for key 16u + 8a' + 4g + b: the A operand (V^T) simply reads
+// its keys in that order.
 //
 // Data movement.  K/V tiles go global -> registers -> LDS, two LDS buffers,
 // one barrier per tile: while tile i is being multiplied, tile i+1 is written
 // to the other buffer, tile i+2 is in flight from HBM and the block-table rows
-// of tile i+3 are being fetched.  K is stored as it lies in memory (row pitch
-// 136 halves); V is stored transposed, V^T[d][key], through an in-register
-// 4x8 transpose (v_perm_b32).  The V^T rows are kept in the order
-// row = 16 * (d % 8) + d / 8 and the thread -> key-quad assignment swaps two
-// index bits, which together make both the 8-byte transposed writes and the
-// 16-byte operand reads free of LDS bank conflicts; as a side effect each lane
-// ends up with runs of 8 consecutive output elements.
+// of tile i+3 are being fetched.  Both tiles are stored row-major as they lie
+// in memory (a thread moves the same four rows of K and of V, so one row
+// lookup serves both).  K rows have a pitch of 136 halves.  V rows have no
+// padding; the four 64-byte chunks of a row are XOR-swizzled with the low two
+// bits of the key instead.  The V^T operand comes out of the row-major tile
+// through ds_read_b64_tr_b16: inside a 16-lane group, lane 4k + r supplies the
+// address of four consecutive head-dim elements of key k and lane j receives
+// element j & 3 of the four lanes {4k' + (j >> 2)}, i.e. one head-dim element
+// of four consecutive keys.  With the swizzle the four key rows a group reads
+// fall into different bank groups, so neither the 16-byte stores nor the
+// transposing reads conflict.  The head-dim order of the A-operand rows is
+// chosen so that each lane ends up with runs of 8 consecutive output elements.
 //
 // Softmax rescaling is lazy: probabilities are taken relative to a per-row
 // reference maximum that is only moved (and O, l rescaled) when the row
@@ -53,9 +62,9 @@ constexpr int kBM = 128;       // query rows per workgroup
 constexpr int kBN = 64;        // keys per tile
 constexpr int kThreads = 256;  // 4 waves
 constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
-constexpr int kVPitch = kBN + 8;       // halves per V^T row in LDS
+constexpr int kVPitch = kHeadDim;      // halves per V row in LDS (chunks swizzled, no padding)
 constexpr int kKTileHalves = kBN * kKPitch;
-constexpr int kVTileHalves = kHeadDim * kVPitch;
+constexpr int kVTileHalves = kBN * kVPitch;
 constexpr size_t kLdsBytes = 2 * size_t(kKTileHalves + kVTileHalves) * sizeof(uint16_t);
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
@@ -118,7 +127,7 @@ template <bool kQF32, bool kOutF32, int kRows>
 __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
     uint16_t* const s_k0 = s_mem;
-    uint16_t* const s_vt0 = s_mem + 2 * kKTileHalves;
+    uint16_t* const s_v0 = s_mem + 2 * kKTileHalves;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
@@ -194,16 +203,16 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[t][r] = 0.0f;
 
-    // ---- tile staging: which rows this thread moves
+    // ---- tile staging: this thread moves 16 bytes of keys ld_r + 16 i, of K and of V
     const uint32_t ld_c = tid & 15;  // 16-byte column of the 256-byte row
     const uint32_t ld_r = tid >> 4;  // 0..15
-    // V: key quad with the two low index bits swapped (see the header comment)
-    const uint32_t v_quad = 4 * (ld_r >> 2) + 2 * (ld_r & 1) + ((ld_r >> 1) & 1);
-    const uint32_t v_col = 16 * (ld_r >> 2) + 8 * ((ld_r >> 1) & 1) + 4 * (ld_r & 1);
+    // V: chunk (ld_c >> 2) of row `key` is stored at chunk (ld_c >> 2) ^ (key & 3); keys
+    // ld_r + 16 i share their low two bits
+    const uint32_t v_st = ld_r * kVPitch + ((((ld_c >> 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
+    const uint32_t k_st = ld_r * kKPitch + 8 * ld_c;
 
     struct TileRows {
-        uint32_t k[4];  // rows of keys ld_r + 16 i
-        uint32_t v[4];  // rows of keys 4 v_quad + i
+        uint32_t r[4];  // rows of keys ld_r + 16 i
     };
     uint4v kreg[4], vreg[4];
 
@@ -213,12 +222,8 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
         const uint32_t last = (seg_b ? len_b : len_a) - 1;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t kk = min(key0 + ld_r + 16 * i, last);
-            const uint32_t vk = min(key0 + 4 * v_quad + i, last);
-            r.k[i] = key_row<kRows>(p, kk, seg_b);
-            r.v[i] = key_row<kRows>(p, vk, seg_b);
-        }
+        for (int i = 0; i < 4; i++)
+            r.r[i] = key_row<kRows>(p, min(key0 + ld_r + 16 * i, last), seg_b);
     };
     auto load_tile = [&](uint32_t it, const TileRows& r) {
         it = min(it, n_tiles - 1);
@@ -228,26 +233,34 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            kreg[i] = *reinterpret_cast<const uint4v*>(kb + int64_t(r.k[i]) * stride);
-            vreg[i] = *reinterpret_cast<const uint4v*>(vb + int64_t(r.v[i]) * stride);
+            const int64_t off = int64_t(r.r[i]) * stride;
+            kreg[i] = *reinterpret_cast<const uint4v*>(kb + off);
+            vreg[i] = *reinterpret_cast<const uint4v*>(vb + off);
         }
     };
     auto store_tile = [&](uint32_t buf) {
-        uint16_t* sk = s_k0 + buf * kKTileHalves;
-        uint16_t* sv = s_vt0 + buf * kVTileHalves;
+        uint16_t* sk = s_k0 + buf * kKTileHalves + k_st;
+        uint16_t* sv = s_v0 + buf * kVTileHalves + v_st;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            *reinterpret_cast<uint4v*>(&sk[(ld_r + 16 * i) * kKPitch + 8 * ld_c]) = kreg[i];
-        // V: 4 keys x 8 d  ->  8 rows of 4 keys; row of d = 8 ld_c + t is 16 t + ld_c
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-            const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
-            uint2v w;
-            w.x = __builtin_amdgcn_perm(vreg[1][t >> 1], vreg[0][t >> 1], sel);
-            w.y = __builtin_amdgcn_perm(vreg[3][t >> 1], vreg[2][t >> 1], sel);
-            *reinterpret_cast<uint2v*>(&sv[(16 * t + ld_c) * kVPitch + v_col]) = w;
+        for (int i = 0; i < 4; i++) {
+            *reinterpret_cast<uint4v*>(sk + 16 * i * kKPitch) = kreg[i];
+            *reinterpret_cast<uint4v*>(sv + 16 * i * kVPitch) = vreg[i];
         }
     };
+
+    // ---- V^T operand reads.  16-lane group q = lane / 16, lane i = 4k + r inside it:
+    // the lane points at key 4 g + k (plus the step's first key), head-dim elements
+    // 32 t + 16 (q & 1) + 8 (r & 1) + 4 (r >> 1) .. + 3, and receives, as row n of the A
+    // operand, one head-dim element of four consecutive keys.
+    uint32_t vt_off[4];  // halves, per head-dim block t
+    {
+        const uint32_t q4 = lane >> 4, i16 = lane & 15;
+        const uint32_t k4 = i16 >> 2, r4 = i16 & 3;
+        const uint32_t key = 4 * g + k4;
+        const uint32_t in_chunk = 16 * (q4 & 1) + 8 * (r4 & 1) + 4 * (r4 >> 1);
+#pragma unroll
+        for (uint32_t t = 0; t < 4; t++) vt_off[t] = key * kVPitch + (((t ^ k4) << 5) | in_chunk);
+    }
 
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
     // ---- prologue: first tile in LDS, second in flight, rows of the third requested
@@ -280,7 +293,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         if (compute) {
             const uint16_t* sk = s_k0 + buf * kKTileHalves;
-            const uint16_t* sv = s_vt0 + buf * kVTileHalves;
+            const uint16_t* sv = s_v0 + buf * kVTileHalves;
 
             // ---- S^T for the two 32-key sub-tiles
             float16v sacc[2];
@@ -311,13 +324,18 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
                     mw1 = w + 1 < p.mask_words ? mask_row[w + 1] : 0u;
                 }
                 const uint32_t limit = diagonal ? min(seg_len, p.start_pos + q_row + 1) : seg_len;
+                // Element r of a sub-tile is key 8 (r >> 2) + (r & 3) + 4 g of it: everything
+                // that depends on the lane goes into `room` and the shifted mask word, the
+                // rest is a compile-time constant (no per-element registers).
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++) {
-                    const uint32_t mw = sub ? mw1 : mw0;
+                    const int32_t room = int32_t(limit) - int32_t(key0 + 32 * sub + 4 * g);
+                    const uint32_t bits = (sub ? mw1 : mw0) >> (4 * g);
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const uint32_t kin = 8 * (r >> 2) + 4 * g + (r & 3);  // key in sub-tile
-                        const bool vis = (key0 + 32 * sub + kin < limit) && ((mw >> kin) & 1u);
+                        constexpr int kDummy = 0;
+                        const int kc = 8 * (r >> 2) + (r & 3) + kDummy;
+                        const bool vis = (room > kc) && ((bits >> kc) & 1u);
                         if (!vis) sacc[sub][r] = -INFINITY;
                     }
                 }
@@ -366,15 +384,20 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                const uint16_t* vrow = &sv[(32 * t + n) * kVPitch + 8 * g];
+                const uint16_t* vbase = sv + vt_off[t];
 #pragma unroll
                 for (int sub = 0; sub < 2; sub++)
 #pragma unroll
                     for (int u = 0; u < 2; u++) {
-                        const half8 a =
-                            as_half8(*reinterpret_cast<const uint4v*>(vrow + 32 * sub + 16 * u));
-                        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp[sub][u], oacc[t],
-                                                                         0, 0, 0);
+                        // keys 32 sub + 16 u + {0, 8} + 4 g + (0..3): k-index 8 g + 4 a' + b
+                        const uint16_t* vp = vbase + (32 * sub + 16 * u) * kVPitch;
+                        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (short4v __attribute__((address_space(3)))*)(vp));
+                        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch));
+                        const short8v a16 = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                            __builtin_bit_cast(half8, a16), bp[sub][u], oacc[t], 0, 0, 0);
                     }
             }
         }
@@ -390,13 +413,13 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const size_t row = (size_t(blockIdx.z) * p.num_heads + head) * p.seq_q + q_row;
         float* po = p.part_o + row * kHeadDim;
 #pragma unroll
-        for (int al = 0; al < 2; al++)
+        for (int t = 0; t < 4; t++)
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
+            for (int ah = 0; ah < 2; ah++) {
                 float x[8];
 #pragma unroll
-                for (int e = 0; e < 8; e++) x[e] = oacc[e >> 1][4 * (al + 2 * (e & 1)) + b];
-                float* op = po + 64 * al + 32 * g + 8 * b;
+                for (int e = 0; e < 8; e++) x[e] = oacc[t][8 * ah + e];
+                float* op = po + 32 * t + 16 * ah + 8 * g;
                 *reinterpret_cast<float4v*>(op) = float4v{x[0], x[1], x[2], x[3]};
                 *reinterpret_cast<float4v*>(op + 4) = float4v{x[4], x[5], x[6], x[7]};
             }
@@ -408,16 +431,17 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     }
     const float inv_l = 1.0f / l_run;
     const int64_t ooff = int64_t(q_row) * p.out_tok_stride + int64_t(head) * p.out_head_stride;
-    // Accumulator [t][4a + b] is LDS row 32t + 8a + 4g + b, i.e. head-dim element
-    // 64 (a & 1) + 32 g + 8 b + 2 t + (a >> 1): 8 consecutive elements per (a & 1, b).
+    // Accumulator [t][4a + b] is A-operand row 8a + 4g + b of block t, which was fed
+    // head-dim element 32 t + 16 (a >> 1) + 8 g + 4 (a & 1) + b: 8 consecutive elements
+    // per (t, a >> 1).
 #pragma unroll
-    for (int al = 0; al < 2; al++)
+    for (int t = 0; t < 4; t++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
+        for (int ah = 0; ah < 2; ah++) {
             float x[8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) x[e] = oacc[e >> 1][4 * (al + 2 * (e & 1)) + b] * inv_l;
-            const uint32_t d = 64 * al + 32 * g + 8 * b;
+            for (int e = 0; e < 8; e++) x[e] = oacc[t][8 * ah + e] * inv_l;
+            const uint32_t d = 32 * t + 16 * ah + 8 * g;
             if constexpr (kOutF32) {
                 float* op = static_cast<float*>(p.out) + ooff + d;
                 *reinterpret_cast<float4v*>(op) = float4v{x[0], x[1], x[2], x[3]};
