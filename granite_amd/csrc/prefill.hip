@@ -10,8 +10,9 @@
 // (fp32 scores and softmax, no epsilon, key k visible iff k <= start_pos + q;
 // tree: cache keys visible, tree key j visible iff j is q or an ancestor).
 //
-// Structure.  grid = (query tiles of 128 rows, query heads); 4 waves, each
-// owning 32 query rows.  Keys are walked in tiles of 64.  Per tile every wave
+// Structure.  grid = (query tiles of 256 rows, query heads, key splits); 8 waves,
+// each owning 32 query rows (one workgroup per CU, two waves per SIMD: a K/V
+// tile staged in LDS serves 256 query rows).  Keys are walked in tiles of 64.  Per tile every wave
 // computes, with v_mfma_f32_32x32x16_f16,
 //
 //   S^T[key, q]  = K[key, :] . Q[q, :]          (A = K from LDS, B = Q in VGPRs)
@@ -58,9 +59,11 @@
 namespace ghip {
 namespace {
 
-constexpr int kBM = 128;       // query rows per workgroup
+constexpr int kBM = 256;       // query rows per workgroup
 constexpr int kBN = 64;        // keys per tile
-constexpr int kThreads = 256;  // 4 waves
+constexpr int kThreads = 512;  // 8 waves, two per SIMD
+constexpr int kStageRows = kThreads / 16;     // key rows moved per staging step
+constexpr int kStageSteps = kBN / kStageRows;  // staging steps per tile
 constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
 constexpr int kVPitch = kHeadDim;      // halves per V row in LDS (chunks swizzled, no padding)
 constexpr int kKTileHalves = kBN * kKPitch;
@@ -203,18 +206,18 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[t][r] = 0.0f;
 
-    // ---- tile staging: this thread moves 16 bytes of keys ld_r + 16 i, of K and of V
+    // ---- tile staging: this thread moves 16 bytes of keys ld_r + kStageRows * i, of K and of V
     const uint32_t ld_c = tid & 15;  // 16-byte column of the 256-byte row
-    const uint32_t ld_r = tid >> 4;  // 0..15
+    const uint32_t ld_r = tid >> 4;  // 0 .. kStageRows - 1
     // V: chunk (ld_c >> 2) of row `key` is stored at chunk (ld_c >> 2) ^ (key & 3); keys
-    // ld_r + 16 i share their low two bits
+    // ld_r + kStageRows * i share their low two bits
     const uint32_t v_st = ld_r * kVPitch + ((((ld_c >> 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
     const uint32_t k_st = ld_r * kKPitch + 8 * ld_c;
 
     struct TileRows {
-        uint32_t r[4];  // rows of keys ld_r + 16 i
+        uint32_t r[kStageSteps];  // rows of keys ld_r + kStageRows * i
     };
-    uint4v kreg[4], vreg[4];
+    uint4v kreg[kStageSteps], vreg[kStageSteps];
 
     auto tile_rows = [&](uint32_t it, TileRows& r) {
         it = min(it, n_tiles - 1);
@@ -222,30 +225,39 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
         const uint32_t last = (seg_b ? len_b : len_a) - 1;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            r.r[i] = key_row<kRows>(p, min(key0 + ld_r + 16 * i, last), seg_b);
+        for (int i = 0; i < kStageSteps; i++)
+            r.r[i] = key_row<kRows>(p, min(key0 + ld_r + kStageRows * i, last), seg_b);
     };
-    auto load_tile = [&](uint32_t it, const TileRows& r) {
+    // K and V of a tile are moved separately: K runs one tile ahead of V (see the loop).
+    auto load_k = [&](uint32_t it, const TileRows& r) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
+        const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
+#pragma unroll
+        for (int i = 0; i < kStageSteps; i++)
+            kreg[i] = *reinterpret_cast<const uint4v*>(kb + int64_t(r.r[i]) * stride);
+    };
+    auto load_v = [&](uint32_t it, const TileRows& r) {
+        it = min(it, n_tiles - 1);
+        const bool seg_b = it >= tiles_a;
         const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int64_t off = int64_t(r.r[i]) * stride;
-            kreg[i] = *reinterpret_cast<const uint4v*>(kb + off);
-            vreg[i] = *reinterpret_cast<const uint4v*>(vb + off);
-        }
+        for (int i = 0; i < kStageSteps; i++)
+            vreg[i] = *reinterpret_cast<const uint4v*>(vb + int64_t(r.r[i]) * stride);
     };
-    auto store_tile = [&](uint32_t buf) {
+    auto store_k = [&](uint32_t buf) {
         uint16_t* sk = s_k0 + buf * kKTileHalves + k_st;
+#pragma unroll
+        for (int i = 0; i < kStageSteps; i++)
+            *reinterpret_cast<uint4v*>(sk + kStageRows * i * kKPitch) = kreg[i];
+    };
+    auto store_v = [&](uint32_t buf) {
         uint16_t* sv = s_v0 + buf * kVTileHalves + v_st;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *reinterpret_cast<uint4v*>(sk + 16 * i * kKPitch) = kreg[i];
-            *reinterpret_cast<uint4v*>(sv + 16 * i * kVPitch) = vreg[i];
-        }
+        for (int i = 0; i < kStageSteps; i++)
+            *reinterpret_cast<uint4v*>(sv + kStageRows * i * kVPitch) = vreg[i];
     };
 
     // ---- V^T operand reads.  16-lane group q = lane / 16, lane i = 4k + r inside it:
@@ -262,144 +274,277 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         for (uint32_t t = 0; t < 4; t++) vt_off[t] = key * kVPitch + (((t ^ k4) << 5) | in_chunk);
     }
 
+    // ---- per-tile pieces
+    struct TileInfo {
+        bool seg_b, active;
+        uint32_t key0, seg_len;
+    };
+    auto tile_info = [&](uint32_t it) -> TileInfo {
+        TileInfo ti;
+        ti.seg_b = it >= tiles_a;
+        ti.key0 = (ti.seg_b ? it - tiles_a : it) * kBN;
+        ti.seg_len = ti.seg_b ? len_b : len_a;
+        ti.active = wave_active && it < n_tiles;
+        if (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !ti.seg_b) {
+            const uint32_t q_last_wave = min(q0 + 32, p.seq_q) - 1;
+            if (ti.key0 > p.start_pos + q_last_wave) ti.active = false;  // nothing visible to this wave
+        }
+        return ti;
+    };
+    // S^T of the 32-key sub-tile `sub` of tile `it` (K in buffer it & 1)
+    auto scores = [&](uint32_t it, int sub, float16v& sacc) {
+        const uint16_t* krow = s_k0 + (it & 1) * kKTileHalves + (32 * sub + n) * kKPitch + 8 * g;
+        float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) {
+            const half8 a = as_half8(*reinterpret_cast<const uint4v*>(krow + 16 * s8));
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[s8], c, 0, 0, 0);
+            if constexpr (kQF32) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[s8], c, 0, 0, 0);
+        }
+        sacc = c;
+    };
+    // Masks of a sub-tile; returns at once on the (common) sub-tiles that need none.
+    auto apply_mask = [&](const TileInfo& ti, int sub, float16v& sacc) {
+        const uint32_t key0 = ti.key0 + 32 * sub;
+        const bool partial = key0 + 32 > ti.seg_len;
+        const bool diagonal = p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !ti.seg_b &&
+                              key0 + 31 > p.start_pos + q0;
+        const bool tree = p.mask_mode == GRANITE_HIP_MASK_TREE && ti.seg_b;
+        if (!(partial || diagonal || tree)) return false;
+        uint32_t mw = 0xFFFFFFFFu;
+        if (tree) {
+            const uint32_t w = key0 >> 5;
+            mw = w < p.mask_words ? mask_row[w] : 0u;
+        }
+        const uint32_t limit = diagonal ? min(ti.seg_len, p.start_pos + q_row + 1) : ti.seg_len;
+        // Element r is key 8 (r >> 2) + (r & 3) + 4 g of the sub-tile: everything that
+        // depends on the lane goes into `room` and the shifted mask word, the rest is
+        // a compile-time constant (no per-element registers).
+        const int32_t room = int32_t(limit) - int32_t(key0 + 4 * g);
+        const uint32_t bits = mw >> (4 * g);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int kc = 8 * (r >> 2) + (r & 3);
+            const bool vis = (room > kc) && ((bits >> kc) & 1u);
+            if (!vis) sacc[r] = -INFINITY;
+        }
+        return true;
+    };
+    // Given the lane's maximum over a sub-tile's scores: the row maximum and, when a row
+    // outgrows the reference maximum, the rescale of m_ref, l and O.
+    auto finish_max = [&](float mraw) {
+        mraw = fmaxf(mraw, wave_shfl_xor(mraw, 32));
+        const float m_tile = mraw * p.scale_log2;
+        if (__any(m_tile > m_ref + kRescaleSlack)) {
+            const float m_new = fmaxf(m_ref, m_tile);
+            const float alpha = fast_exp2(m_ref - m_new);
+            m_ref = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
+        }
+    };
+    auto mask_and_max = [&](const TileInfo& ti, int sub, float16v& sacc) {
+        apply_mask(ti, sub, sacc);
+        float mraw = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
+        finish_max(mraw);
+    };
+    // P^T = exp2(S^T * scale - m_ref) of a sub-tile as B operands of the second product;
+    // adds to l.
+    auto probabilities = [&](const float16v& sacc, half8 (&bp)[2]) {
+        float psum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            float pe[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                pe[j] = fast_exp2(__builtin_fmaf(sacc[8 * u + j], p.scale_log2, -m_ref));
+                psum += pe[j];
+            }
+            uint4v w;
+            w.x = pack_f16x2(pe[0], pe[1]);
+            w.y = pack_f16x2(pe[2], pe[3]);
+            w.z = pack_f16x2(pe[4], pe[5]);
+            w.w = pack_f16x2(pe[6], pe[7]);
+            bp[u] = as_half8(w);
+        }
+        l_run += psum;
+    };
+    // O^T += V^T P^T for sub-tile `sub` of tile `it` (V in buffer it & 1)
+    auto accumulate = [&](uint32_t it, int sub, const half8 (&bp)[2]) {
+        const uint16_t* sv = s_v0 + (it & 1) * kVTileHalves + 32 * sub * kVPitch;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                // keys 16 u + {0, 8} + 4 g + (0..3) of the sub-tile: k-index 8 g + 4 a' + b
+                const uint16_t* vp = sv + vt_off[t] + 16 * u * kVPitch;
+                const uint2v lo = __builtin_bit_cast(
+                    uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (short4v __attribute__((address_space(3)))*)(vp)));
+                const uint2v hi = __builtin_bit_cast(
+                    uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch)));
+                const uint4v a16 = {lo.x, lo.y, hi.x, hi.y};
+                oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(a16), bp[u], oacc[t], 0,
+                                                                 0, 0);
+            }
+        }
+    };
+
+    // One pipeline phase with the two instruction streams interleaved by hand: the 8
+    // MFMAs of the scores of sub-tile (it_q, sub_q), each followed by a slice of the softmax
+    // arithmetic of the previous sub-tile (scores s_in), then the 8 MFMAs of the second
+    // product for (it_v, sub_v).  On this part a 32x32x16 MFMA keeps the vector ALU to
+    // itself for only half of its 32 cycles and transcendentals run beside it, so vector
+    // work placed between MFMAs is nearly free, while vector work after a burst of MFMAs
+    // is not; the scheduling barriers keep the compiler from regrouping the slices.
+    // Operands are fetched from LDS two steps ahead.
+    auto fused_phase = [&](const TileInfo& ti_q, uint32_t it_q, int sub_q, float16v& s_out,
+                           const float16v& s_in, uint32_t it_v, int sub_v) {
+        const uint16_t* krow =
+            s_k0 + (it_q & 1) * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
+        const uint16_t* sv = s_v0 + (it_v & 1) * kVTileHalves + 32 * sub_v * kVPitch;
+        auto k_operand = [&](int s8) -> uint4v {
+            return *reinterpret_cast<const uint4v*>(krow + 16 * s8);
+        };
+        auto v_operand = [&](int i) -> uint4v {  // step i: head-dim block i & 3, key half i >> 2
+            const uint16_t* vp = sv + vt_off[i & 3] + 16 * (i >> 2) * kVPitch;
+            const uint2v lo = __builtin_bit_cast(
+                uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (short4v __attribute__((address_space(3)))*)(vp)));
+            const uint2v hi = __builtin_bit_cast(
+                uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch)));
+            return uint4v{lo.x, lo.y, hi.x, hi.y};
+        };
+        uint4v ring[3];
+        ring[0] = k_operand(0);
+        ring[1] = k_operand(1);
+        float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        float psum = 0.0f;
+        uint32_t pw[8];
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) {
+#ifdef GHIP_EXP_NO_QK
+            c[s8] += bq[s8][0];
+#else
+            if (s8 + 2 < 8) ring[(s8 + 2) % 3] = k_operand(s8 + 2);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % 3]), bq[s8], c, 0, 0, 0);
+#endif
+            if constexpr (kQF32)
+                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % 3]), bq_lo[s8], c, 0, 0, 0);
+#ifdef GHIP_EXP_NO_SOFTMAX
+            const float e0 = s_in[2 * s8], e1 = s_in[2 * s8 + 1];
+#else
+            const float e0 = fast_exp2(__builtin_fmaf(s_in[2 * s8], p.scale_log2, -m_ref));
+            const float e1 = fast_exp2(__builtin_fmaf(s_in[2 * s8 + 1], p.scale_log2, -m_ref));
+            psum += e0;
+            psum += e1;
+#endif
+            pw[s8] = pack_f16x2(e0, e1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        l_run += psum;
+        const half8 bp0 = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
+        const half8 bp1 = as_half8(uint4v{pw[4], pw[5], pw[6], pw[7]});
+        ring[0] = v_operand(0);
+        ring[1] = v_operand(1);
+        apply_mask(ti_q, sub_q, c);  // rare; the maximum of the new scores rides along below
+        float mraw = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            mraw = fmaxf(fmaxf(mraw, c[2 * i]), c[2 * i + 1]);
+#ifdef GHIP_EXP_NO_PV
+            oacc[i & 3][i] += float(((i >> 2) ? bp1 : bp0)[0]);
+#else
+            if (i + 2 < 8) ring[(i + 2) % 3] = v_operand(i + 2);
+            oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % 3]),
+                                                                 (i >> 2) ? bp1 : bp0, oacc[i & 3], 0, 0, 0);
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        s_out = c;
+        finish_max(mraw);
+    };
+
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
-    // ---- prologue: first tile in LDS, second in flight, rows of the third requested
-    TileRows rows;
-    tile_rows(t_begin, rows);
-    load_tile(t_begin, rows);
-    tile_rows(t_begin + 1, rows);
-    store_tile(t_begin & 1);
-    load_tile(t_begin + 1, rows);
-    tile_rows(t_begin + 2, rows);
+    // ---- prologue.  In LDS: K of the first two tiles, V of the first.  In flight: K of the
+    // third tile, V of the second.  Row lookups: one tile further.
+    TileRows rows_v, rows_k;  // rows of the tiles whose V / K is loaded next
+    tile_rows(t_begin, rows_k);
+    load_k(t_begin, rows_k);
+    load_v(t_begin, rows_k);
+    tile_rows(t_begin + 1, rows_v);
+    store_k(t_begin & 1);
+    store_v(t_begin & 1);
+    load_k(t_begin + 1, rows_v);
+    tile_rows(t_begin + 2, rows_k);
+    store_k((t_begin + 1) & 1);
+    load_v(t_begin + 1, rows_v);
+    load_k(t_begin + 2, rows_k);
+    rows_v = rows_k;
+    tile_rows(t_begin + 3, rows_k);
     __syncthreads();
 
-    for (uint32_t it = t_begin; it < n_tiles; it++) {
-        const uint32_t buf = it & 1;
-        // Unconditional (indices clamp at the last tile): loads inside a branch would
-        // force a full wait at the join.  The extra store after the last tile goes to the
-        // buffer nobody reads any more.
-        store_tile(buf ^ 1);      // tile it+1 (arrived during the previous tile)
-        load_tile(it + 2, rows);  // tile it+2 flies during this tile's math
-        tile_rows(it + 3, rows);
-
-        const bool seg_b = it >= tiles_a;
-        const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
-        const uint32_t seg_len = seg_b ? len_b : len_a;
-
-        bool compute = wave_active;
-        if (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !seg_b) {
-            const uint32_t q_last_wave = min(q0 + 32, p.seq_q) - 1;
-            if (key0 > p.start_pos + q_last_wave) compute = false;
+    // The loop is software pipelined over 32-key sub-tiles: while the vector ALU turns
+    // the scores of one sub-tile into probabilities, the matrix pipe already computes the
+    // scores of the next one, and the maximum of those is taken while the second product
+    // of the current sub-tile runs.  s0 holds the scores of sub-tile 0 of the current tile
+    // on entry to an iteration; K is therefore staged one tile ahead of V.
+    float16v s0, s1;
+    {
+        const TileInfo first = tile_info(t_begin);
+        if (first.active) {
+            scores(t_begin, 0, s0);
+            mask_and_max(first, 0, s0);
         }
-        if (compute) {
-            const uint16_t* sk = s_k0 + buf * kKTileHalves;
-            const uint16_t* sv = s_v0 + buf * kVTileHalves;
+    }
+    for (uint32_t it = t_begin; it < n_tiles; it++) {
+        // Unconditional staging (indices clamp at the last tile): loads inside a branch
+        // would force a full wait at the join.  Stores past the last tile go to buffers
+        // nobody reads any more.
+#ifndef GHIP_EXP_NO_LSTORE
+        store_v((it + 1) & 1);  // V of tile it + 1
+#endif
+#ifndef GHIP_EXP_NO_GLOAD
+        load_v(it + 2, rows_v);
+#endif
+        rows_v = rows_k;
 
-            // ---- S^T for the two 32-key sub-tiles
-            float16v sacc[2];
-#pragma unroll
-            for (int sub = 0; sub < 2; sub++) {
-                const uint16_t* krow = &sk[(32 * sub + n) * kKPitch + 8 * g];
-                float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-                for (int s = 0; s < 8; s++) {
-                    const half8 a = as_half8(*reinterpret_cast<const uint4v*>(krow + 16 * s));
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[s], c, 0, 0, 0);
-                    if constexpr (kQF32)
-                        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[s], c, 0, 0, 0);
-                }
-                sacc[sub] = c;
+        const TileInfo cur = tile_info(it);
+        const TileInfo nxt = tile_info(it + 1);
+        half8 bp[2];
+        // phase A: last use of K of tile it
+        if (cur.active) {
+            fused_phase(cur, it, 1, s1, s0, it, 0);
+        }
+#ifndef GHIP_EXP_ONE_BARRIER
+        __syncthreads();
+#endif
+#ifndef GHIP_EXP_NO_LSTORE
+        store_k(it & 1);  // K of tile it + 2 replaces K of tile it
+#endif
+#ifndef GHIP_EXP_NO_GLOAD
+        load_k(it + 3, rows_k);
+#endif
+#ifndef GHIP_EXP_NO_ROWS
+        tile_rows(it + 4, rows_k);
+#endif
+        // phase B
+        if (cur.active && nxt.active) {  // the common case, in one block for the scheduler
+            fused_phase(nxt, it + 1, 0, s0, s1, it, 1);
+        } else {
+            if (nxt.active) scores(it + 1, 0, s0);
+            if (cur.active) {
+                probabilities(s1, bp);
+                accumulate(it, 1, bp);
             }
-
-            // ---- masks (only on tiles that need them)
-            const bool partial = key0 + kBN > seg_len;
-            const bool diagonal = p.mask_mode == GRANITE_HIP_MASK_CAUSAL && !seg_b &&
-                                  key0 + kBN - 1 > p.start_pos + q0;
-            const bool tree = p.mask_mode == GRANITE_HIP_MASK_TREE && seg_b;
-            if (partial || diagonal || tree) {
-                uint32_t mw0 = 0xFFFFFFFFu, mw1 = 0xFFFFFFFFu;
-                if (tree) {
-                    const uint32_t w = key0 >> 5;
-                    mw0 = w < p.mask_words ? mask_row[w] : 0u;
-                    mw1 = w + 1 < p.mask_words ? mask_row[w + 1] : 0u;
-                }
-                const uint32_t limit = diagonal ? min(seg_len, p.start_pos + q_row + 1) : seg_len;
-                // Element r of a sub-tile is key 8 (r >> 2) + (r & 3) + 4 g of it: everything
-                // that depends on the lane goes into `room` and the shifted mask word, the
-                // rest is a compile-time constant (no per-element registers).
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++) {
-                    const int32_t room = int32_t(limit) - int32_t(key0 + 32 * sub + 4 * g);
-                    const uint32_t bits = (sub ? mw1 : mw0) >> (4 * g);
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        constexpr int kDummy = 0;
-                        const int kc = 8 * (r >> 2) + (r & 3) + kDummy;
-                        const bool vis = (room > kc) && ((bits >> kc) & 1u);
-                        if (!vis) sacc[sub][r] = -INFINITY;
-                    }
-                }
-            }
-
-            // ---- softmax relative to m_ref; move m_ref only when a row outgrows it
-            float mraw = -INFINITY;
-#pragma unroll
-            for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[sub][r]);
-            mraw = fmaxf(mraw, wave_shfl_xor(mraw, 32));
-            const float m_tile = mraw * p.scale_log2;
-            if (__any(m_tile > m_ref + kRescaleSlack)) {
-                const float m_new = fmaxf(m_ref, m_tile);
-                const float alpha = fast_exp2(m_ref - m_new);
-                m_ref = m_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
-            }
-            float psum = 0.0f;
-            half8 bp[2][2];
-#pragma unroll
-            for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    float pe[8];
-#pragma unroll
-                    for (int j = 0; j < 8; j++) {
-                        pe[j] =
-                            fast_exp2(__builtin_fmaf(sacc[sub][8 * u + j], p.scale_log2, -m_ref));
-                        psum += pe[j];
-                    }
-                    uint4v w;
-                    w.x = pack_f16x2(pe[0], pe[1]);
-                    w.y = pack_f16x2(pe[2], pe[3]);
-                    w.z = pack_f16x2(pe[4], pe[5]);
-                    w.w = pack_f16x2(pe[6], pe[7]);
-                    bp[sub][u] = as_half8(w);
-                }
-            l_run += psum;
-
-            // ---- O^T += V^T P^T
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const uint16_t* vbase = sv + vt_off[t];
-#pragma unroll
-                for (int sub = 0; sub < 2; sub++)
-#pragma unroll
-                    for (int u = 0; u < 2; u++) {
-                        // keys 32 sub + 16 u + {0, 8} + 4 g + (0..3): k-index 8 g + 4 a' + b
-                        const uint16_t* vp = vbase + (32 * sub + 16 * u) * kVPitch;
-                        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (short4v __attribute__((address_space(3)))*)(vp));
-                        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch));
-                        const short8v a16 = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                            __builtin_bit_cast(half8, a16), bp[sub][u], oacc[t], 0, 0, 0);
-                    }
-            }
+            if (nxt.active) mask_and_max(nxt, 0, s0);
         }
         __syncthreads();
     }
@@ -621,14 +766,14 @@ int launch_attention(const granite_hip_attention_args& a) {
     if (q_tiles > 0x7FFFFFFFu / 2 || a.num_heads > 65535u) return GRANITE_HIP_EINVAL;
 
     // Split the keys over several workgroups when (query tiles x heads) alone cannot
-    // put two workgroups on every CU; every split keeps at least 4 key tiles.
+    // put a workgroup on every CU; every split keeps at least 4 key tiles.
     uint32_t n_splits = 1;
     {
         const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
         const uint64_t wgs = uint64_t(q_tiles) * a.num_heads;
         const uint32_t key_tiles = (a.cache_len + kBN - 1) / kBN + (a.extra_len + kBN - 1) / kBN;
-        if (wgs < 2 * cus) {
-            n_splits = uint32_t((2 * cus + wgs - 1) / wgs);
+        if (wgs < cus) {
+            n_splits = uint32_t((cus + wgs - 1) / wgs);
             n_splits = min(n_splits, max(key_tiles / 4, 1u));
             n_splits = min(n_splits, 64u);
         }
