@@ -120,6 +120,21 @@ __device__ __forceinline__ float wave_shfl_xor(float v, int mask) {
     return __shfl_xor(v, mask, kWave);
 }
 
+// The values of lanes l and l ^ 32 side by side, through v_permlane32_swap (one vector
+// instruction, no LDS round trip): .lo is the value held by the lane's copy in lanes
+// 0..31, .hi that of its copy in lanes 32..63; both lanes see the same pair.  Written as
+// inline assembly because the compiler builtin loses the second result when both
+// operands carry the same value.  The s_nop covers the two wait states the instruction
+// needs after a vector write to its operands.
+struct LanePair {
+    float lo, hi;
+};
+__device__ __forceinline__ LanePair half_wave_pair(float v) {
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return LanePair{a, b};
+}
+
 #endif  // __HIPCC__
 
 }  // namespace ghip

@@ -68,7 +68,8 @@ constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
 constexpr int kVPitch = kHeadDim;      // halves per V row in LDS (chunks swizzled, no padding)
 constexpr int kKTileHalves = kBN * kKPitch;
 constexpr int kVTileHalves = kBN * kVPitch;
-constexpr size_t kLdsBytes = 2 * size_t(kKTileHalves + kVTileHalves) * sizeof(uint16_t);
+constexpr int kKBuffers = 3;  // K runs a tile ahead of V and is read across two iterations
+constexpr size_t kLdsBytes = size_t(kKBuffers * kKTileHalves + 2 * kVTileHalves) * sizeof(uint16_t);
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -130,7 +131,7 @@ template <bool kQF32, bool kOutF32, int kRows>
 __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
     uint16_t* const s_k0 = s_mem;
-    uint16_t* const s_v0 = s_mem + 2 * kKTileHalves;
+    uint16_t* const s_v0 = s_mem + kKBuffers * kKTileHalves;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
@@ -291,9 +292,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         return ti;
     };
-    // S^T of the 32-key sub-tile `sub` of tile `it` (K in buffer it & 1)
-    auto scores = [&](uint32_t it, int sub, float16v& sacc) {
-        const uint16_t* krow = s_k0 + (it & 1) * kKTileHalves + (32 * sub + n) * kKPitch + 8 * g;
+    // S^T of the 32-key sub-tile `sub` of the tile whose K is in buffer `kbuf`
+    auto scores = [&](uint32_t kbuf, int sub, float16v& sacc) {
+        const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub + n) * kKPitch + 8 * g;
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++) {
@@ -333,8 +334,8 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     // Given the lane's maximum over a sub-tile's scores: the row maximum and, when a row
     // outgrows the reference maximum, the rescale of m_ref, l and O.
     auto finish_max = [&](float mraw) {
-        mraw = fmaxf(mraw, wave_shfl_xor(mraw, 32));
-        const float m_tile = mraw * p.scale_log2;
+        const LanePair both = half_wave_pair(mraw);
+        const float m_tile = fmaxf(both.lo, both.hi) * p.scale_log2;
         if (__any(m_tile > m_ref + kRescaleSlack)) {
             const float m_new = fmaxf(m_ref, m_tile);
             const float alpha = fast_exp2(m_ref - m_new);
@@ -374,9 +375,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         l_run += psum;
     };
-    // O^T += V^T P^T for sub-tile `sub` of tile `it` (V in buffer it & 1)
-    auto accumulate = [&](uint32_t it, int sub, const half8 (&bp)[2]) {
-        const uint16_t* sv = s_v0 + (it & 1) * kVTileHalves + 32 * sub * kVPitch;
+    // O^T += V^T P^T for sub-tile `sub` of the tile whose V is in buffer `vbuf`
+    auto accumulate = [&](uint32_t vbuf, int sub, const half8 (&bp)[2]) {
+        const uint16_t* sv = s_v0 + vbuf * kVTileHalves + 32 * sub * kVPitch;
 #pragma unroll
         for (int t = 0; t < 4; t++) {
 #pragma unroll
@@ -404,11 +405,10 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     // work placed between MFMAs is nearly free, while vector work after a burst of MFMAs
     // is not; the scheduling barriers keep the compiler from regrouping the slices.
     // Operands are fetched from LDS two steps ahead.
-    auto fused_phase = [&](const TileInfo& ti_q, uint32_t it_q, int sub_q, float16v& s_out,
-                           const float16v& s_in, uint32_t it_v, int sub_v) {
-        const uint16_t* krow =
-            s_k0 + (it_q & 1) * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
-        const uint16_t* sv = s_v0 + (it_v & 1) * kVTileHalves + 32 * sub_v * kVPitch;
+    auto fused_phase = [&](const TileInfo& ti_q, uint32_t kbuf, int sub_q, float16v& s_out,
+                           const float16v& s_in, uint32_t it_v /* V buffer */, int sub_v) {
+        const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
+        const uint16_t* sv = s_v0 + it_v * kVTileHalves + 32 * sub_v * kVPitch;
         auto k_operand = [&](int s8) -> uint4v {
             return *reinterpret_cast<const uint4v*>(krow + 16 * s8);
         };
@@ -422,38 +422,59 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
                             (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch)));
             return uint4v{lo.x, lo.y, hi.x, hi.y};
         };
-        uint4v ring[3];
-        ring[0] = k_operand(0);
-        ring[1] = k_operand(1);
+#ifdef GHIP_EXP_RING4
+        constexpr int kRing = 4;
+#else
+        constexpr int kRing = 3;
+#endif
+        uint4v ring[kRing];
+#pragma unroll
+        for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(i);
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         float psum = 0.0f;
         uint32_t pw[8];
+        // The softmax slices are themselves pipelined over the steps, so that no step
+        // waits on its own results: step s8 scales the scores of slice s8 + 1, takes the
+        // exponentials of slice s8 and sums and packs slice s8 - 1.
+        float t0 = __builtin_fmaf(s_in[0], p.scale_log2, -m_ref);
+        float t1 = __builtin_fmaf(s_in[1], p.scale_log2, -m_ref);
+        float ep0 = 0.0f, ep1 = 0.0f;
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++) {
 #ifdef GHIP_EXP_NO_QK
             c[s8] += bq[s8][0];
 #else
-            if (s8 + 2 < 8) ring[(s8 + 2) % 3] = k_operand(s8 + 2);
-            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % 3]), bq[s8], c, 0, 0, 0);
+            if (s8 + kRing - 1 < 8) ring[(s8 + kRing - 1) % kRing] = k_operand(s8 + kRing - 1);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq[s8], c, 0, 0, 0);
 #endif
             if constexpr (kQF32)
-                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % 3]), bq_lo[s8], c, 0, 0, 0);
-#ifdef GHIP_EXP_NO_SOFTMAX
-            const float e0 = s_in[2 * s8], e1 = s_in[2 * s8 + 1];
-#else
-            const float e0 = fast_exp2(__builtin_fmaf(s_in[2 * s8], p.scale_log2, -m_ref));
-            const float e1 = fast_exp2(__builtin_fmaf(s_in[2 * s8 + 1], p.scale_log2, -m_ref));
-            psum += e0;
-            psum += e1;
-#endif
-            pw[s8] = pack_f16x2(e0, e1);
+                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq_lo[s8], c, 0, 0, 0);
+            const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
+            if (s8 < 7) {
+                t0 = __builtin_fmaf(s_in[2 * s8 + 2], p.scale_log2, -m_ref);
+                t1 = __builtin_fmaf(s_in[2 * s8 + 3], p.scale_log2, -m_ref);
+            }
+            if (s8 > 0) {
+                psum += ep0;
+                psum += ep1;
+                pw[s8 - 1] = pack_f16x2(ep0, ep1);
+            }
+            ep0 = e0;
+            ep1 = e1;
+            // pin the slice here: without it the optimiser sinks the softmax arithmetic
+            // below the (rarely taken) mask branch, away from the MFMAs it should hide behind
+            asm volatile("" : "+v"(ep0), "+v"(ep1), "+v"(t0), "+v"(t1), "+v"(psum));
+            if (s8 > 0) asm volatile("" : "+v"(pw[s8 - 1]));
             __builtin_amdgcn_sched_barrier(0);
         }
+        psum += ep0;
+        psum += ep1;
+        pw[7] = pack_f16x2(ep0, ep1);
         l_run += psum;
         const half8 bp0 = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
         const half8 bp1 = as_half8(uint4v{pw[4], pw[5], pw[6], pw[7]});
-        ring[0] = v_operand(0);
-        ring[1] = v_operand(1);
+#pragma unroll
+        for (int i = 0; i < kRing - 1; i++) ring[i] = v_operand(i);
         apply_mask(ti_q, sub_q, c);  // rare; the maximum of the new scores rides along below
         float mraw = -INFINITY;
 #pragma unroll
@@ -462,8 +483,8 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
 #ifdef GHIP_EXP_NO_PV
             oacc[i & 3][i] += float(((i >> 2) ? bp1 : bp0)[0]);
 #else
-            if (i + 2 < 8) ring[(i + 2) % 3] = v_operand(i + 2);
-            oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % 3]),
+            if (i + kRing - 1 < 8) ring[(i + kRing - 1) % kRing] = v_operand(i + kRing - 1);
+            oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % kRing]),
                                                                  (i >> 2) ? bp1 : bp0, oacc[i & 3], 0, 0, 0);
 #endif
             __builtin_amdgcn_sched_barrier(0);
@@ -475,16 +496,17 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
     // ---- prologue.  In LDS: K of the first two tiles, V of the first.  In flight: K of the
     // third tile, V of the second.  Row lookups: one tile further.
+    // K of tile t_begin + j lives in buffer j % 3, V in buffer j & 1.
     TileRows rows_v, rows_k;  // rows of the tiles whose V / K is loaded next
     tile_rows(t_begin, rows_k);
     load_k(t_begin, rows_k);
     load_v(t_begin, rows_k);
     tile_rows(t_begin + 1, rows_v);
-    store_k(t_begin & 1);
-    store_v(t_begin & 1);
+    store_k(0);
+    store_v(0);
     load_k(t_begin + 1, rows_v);
     tile_rows(t_begin + 2, rows_k);
-    store_k((t_begin + 1) & 1);
+    store_k(1);
     load_v(t_begin + 1, rows_v);
     load_k(t_begin + 2, rows_k);
     rows_v = rows_k;
@@ -495,63 +517,65 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     // the scores of one sub-tile into probabilities, the matrix pipe already computes the
     // scores of the next one, and the maximum of those is taken while the second product
     // of the current sub-tile runs.  s0 holds the scores of sub-tile 0 of the current tile
-    // on entry to an iteration; K is therefore staged one tile ahead of V.
+    // on entry to an iteration; K is therefore staged one tile ahead of V and kept in three
+    // buffers (the tile being finished, the next one, the one being written), which leaves
+    // one barrier per tile.
     float16v s0, s1;
     {
         const TileInfo first = tile_info(t_begin);
         if (first.active) {
-            scores(t_begin, 0, s0);
+            scores(0, 0, s0);
             mask_and_max(first, 0, s0);
         }
     }
+    uint32_t kb_cur = 0, kb_next = 1, kb_store = 2;  // K buffers of tiles it, it + 1, it + 2
+    uint32_t vb_cur = 0;                              // V buffer of tile it
     for (uint32_t it = t_begin; it < n_tiles; it++) {
         // Unconditional staging (indices clamp at the last tile): loads inside a branch
         // would force a full wait at the join.  Stores past the last tile go to buffers
         // nobody reads any more.
 #ifndef GHIP_EXP_NO_LSTORE
-        store_v((it + 1) & 1);  // V of tile it + 1
+        store_k(kb_store);     // K of tile it + 2
+        store_v(vb_cur ^ 1);   // V of tile it + 1
 #endif
 #ifndef GHIP_EXP_NO_GLOAD
+        load_k(it + 3, rows_k);
         load_v(it + 2, rows_v);
 #endif
         rows_v = rows_k;
+#ifndef GHIP_EXP_NO_ROWS
+        tile_rows(it + 4, rows_k);
+#endif
 
         const TileInfo cur = tile_info(it);
         const TileInfo nxt = tile_info(it + 1);
         half8 bp[2];
-        // phase A: last use of K of tile it
-        if (cur.active) {
-            fused_phase(cur, it, 1, s1, s0, it, 0);
-        }
-#ifndef GHIP_EXP_ONE_BARRIER
-        __syncthreads();
-#endif
-#ifndef GHIP_EXP_NO_LSTORE
-        store_k(it & 1);  // K of tile it + 2 replaces K of tile it
-#endif
-#ifndef GHIP_EXP_NO_GLOAD
-        load_k(it + 3, rows_k);
-#endif
-#ifndef GHIP_EXP_NO_ROWS
-        tile_rows(it + 4, rows_k);
-#endif
-        // phase B
-        if (cur.active && nxt.active) {  // the common case, in one block for the scheduler
-            fused_phase(nxt, it + 1, 0, s0, s1, it, 1);
+        if (cur.active && nxt.active) {  // the common case
+            fused_phase(cur, kb_cur, 1, s1, s0, vb_cur, 0);
+            fused_phase(nxt, kb_next, 0, s0, s1, vb_cur, 1);
         } else {
-            if (nxt.active) scores(it + 1, 0, s0);
+            if (cur.active) fused_phase(cur, kb_cur, 1, s1, s0, vb_cur, 0);
+            if (nxt.active) scores(kb_next, 0, s0);
             if (cur.active) {
                 probabilities(s1, bp);
-                accumulate(it, 1, bp);
+                accumulate(vb_cur, 1, bp);
             }
             if (nxt.active) mask_and_max(nxt, 0, s0);
         }
         __syncthreads();
+        const uint32_t freed = kb_cur;
+        kb_cur = kb_next;
+        kb_next = kb_store;
+        kb_store = freed;
+        vb_cur ^= 1;
     }
     }
 
     if (!wave_active) return;
-    l_run += wave_shfl_xor(l_run, 32);
+    {
+        const LanePair both = half_wave_pair(l_run);
+        l_run = both.lo + both.hi;
+    }
     if (q_row >= p.seq_q) return;
     if (gridDim.z > 1) {
         // partial result of this key range: O unnormalised, (m_ref, l) beside it
