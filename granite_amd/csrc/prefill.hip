@@ -62,14 +62,14 @@ namespace {
 constexpr int kBM = 256;       // query rows per workgroup
 constexpr int kBN = 64;        // keys per tile
 constexpr int kThreads = 512;  // 8 waves, two per SIMD
-constexpr int kStageRows = kThreads / 16;     // key rows moved per staging step
-constexpr int kStageSteps = kBN / kStageRows;  // staging steps per tile
 constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
 constexpr int kVPitch = kHeadDim;      // halves per V row in LDS (chunks swizzled, no padding)
 constexpr int kKTileHalves = kBN * kKPitch;
 constexpr int kVTileHalves = kBN * kVPitch;
 constexpr int kKBuffers = 3;  // K runs a tile ahead of V and is read across two iterations
-constexpr size_t kLdsBytes = size_t(kKBuffers * kKTileHalves + 2 * kVTileHalves) * sizeof(uint16_t);
+constexpr int kVBuffers = 3;  // V of the previous tile is still read while the next is written
+constexpr size_t kLdsBytes =
+    size_t(kKBuffers * kKTileHalves + kVBuffers * kVTileHalves) * sizeof(uint16_t);
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -97,7 +97,8 @@ struct AttnParams {
     int mask_mode;
     uint32_t start_pos, seq_q, num_heads, group;
     float scale_log2;
-    // split-K over the key tiles (gridDim.z > 1): unnormalised partial results
+    uint32_t q_tiles, n_splits;  // the grid: q_tiles * num_heads * n_splits workgroups
+    // split-K over the key tiles (n_splits > 1): unnormalised partial results
     float* part_o;   // [split, head, q, D]
     float* part_ml;  // [split, head, q, 2] = (reference max, sum)
     void* final_out;
@@ -139,9 +140,23 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     const uint32_t n = lane & 31;  // query row inside the wave / MFMA row index m
     const uint32_t g = lane >> 5;  // MFMA k-group (0/1)
 
+    // ---- which (query tile, head, key split) this workgroup computes.  Workgroups are
+    // handed to the 8 XCDs round-robin by their linear id, and every XCD has its own L2;
+    // the ids are therefore remapped so that an XCD receives a contiguous run of the list
+    // ordered (kv head, split, head in group, query tile): the workgroups that stream the
+    // same K/V range share an L2 instead of fetching it once per XCD.
+    uint32_t job = blockIdx.x;
+    {
+        constexpr uint32_t kXcds = 8;
+        const uint32_t total = gridDim.x;
+        if (total % kXcds == 0) job = (job % kXcds) * (total / kXcds) + job / kXcds;
+    }
+    const uint32_t members = p.group * p.q_tiles;  // workgroups per (kv head, split)
+    const uint32_t gidx = job / members, member = job - gidx * members;
+    const uint32_t split = gidx % p.n_splits;
+    const uint32_t head = (gidx / p.n_splits) * p.group + member / p.q_tiles;
     // heavy (late) query tiles first so the causal tail is short
-    const uint32_t q_tile = gridDim.x - 1 - blockIdx.x;
-    const uint32_t head = blockIdx.y;
+    const uint32_t q_tile = p.q_tiles - 1 - member % p.q_tiles;
     const uint32_t kvh = head / p.group;
     const uint32_t q0_wg = q_tile * kBM;
     const uint32_t q0 = q0_wg + 32 * wave;
@@ -159,9 +174,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     const uint32_t tiles_a = (len_a + kBN - 1) / kBN;
     const uint32_t tiles_b = (len_b + kBN - 1) / kBN;
     const uint32_t all_tiles = tiles_a + tiles_b;
-    // this workgroup's share of the key tiles when the keys are split over gridDim.z
-    const uint32_t t_begin = uint32_t(uint64_t(all_tiles) * blockIdx.z / gridDim.z);
-    const uint32_t n_tiles = uint32_t(uint64_t(all_tiles) * (blockIdx.z + 1) / gridDim.z);
+    // this workgroup's share of the key tiles when the keys are split
+    const uint32_t t_begin = uint32_t(uint64_t(all_tiles) * split / p.n_splits);
+    const uint32_t n_tiles = uint32_t(uint64_t(all_tiles) * (split + 1) / p.n_splits);
 
     const uint16_t* ka_base = p.k + size_t(kvh) * p.a_head_stride;
     const uint16_t* va_base = p.v + size_t(kvh) * p.a_head_stride;
@@ -207,27 +222,29 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[t][r] = 0.0f;
 
-    // ---- tile staging: this thread moves 16 bytes of keys ld_r + kStageRows * i, of K and of V
-    const uint32_t ld_c = tid & 15;  // 16-byte column of the 256-byte row
-    const uint32_t ld_r = tid >> 4;  // 0 .. kStageRows - 1
-    // V: chunk (ld_c >> 2) of row `key` is stored at chunk (ld_c >> 2) ^ (key & 3); keys
-    // ld_r + kStageRows * i share their low two bits
+    // ---- tile staging: this thread moves two 16-byte pieces of key ld_r, columns ld_c and
+    // ld_c + 8 of the 256-byte row, of K and of V: one row lookup and one address per
+    // thread and tile, and every load instruction still covers whole 128-byte lines.
+    static_assert(kThreads == 8 * kBN, "two 16-byte pieces of one row per thread");
+    const uint32_t ld_c = tid & 7;   // 16-byte column of the first piece
+    const uint32_t ld_r = tid >> 3;  // key inside the tile, 0 .. 63
+    // V: chunk (col >> 2) of row `key` is stored at chunk (col >> 2) ^ (key & 3); the second
+    // piece is two chunks further
     const uint32_t v_st = ld_r * kVPitch + ((((ld_c >> 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
+    const uint32_t v_st2 = ld_r * kVPitch + (((((ld_c >> 2) + 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
     const uint32_t k_st = ld_r * kKPitch + 8 * ld_c;
 
     struct TileRows {
-        uint32_t r[kStageSteps];  // rows of keys ld_r + kStageRows * i
+        uint32_t r;  // row of key ld_r
     };
-    uint4v kreg[kStageSteps], vreg[kStageSteps];
+    uint4v kreg[2], vreg[2];
 
     auto tile_rows = [&](uint32_t it, TileRows& r) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
         const uint32_t last = (seg_b ? len_b : len_a) - 1;
-#pragma unroll
-        for (int i = 0; i < kStageSteps; i++)
-            r.r[i] = key_row<kRows>(p, min(key0 + ld_r + kStageRows * i, last), seg_b);
+        r.r = key_row<kRows>(p, min(key0 + ld_r, last), seg_b);
     };
     // K and V of a tile are moved separately: K runs one tile ahead of V (see the loop).
     auto load_k = [&](uint32_t it, const TileRows& r) {
@@ -235,30 +252,28 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const bool seg_b = it >= tiles_a;
         const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
-#pragma unroll
-        for (int i = 0; i < kStageSteps; i++)
-            kreg[i] = *reinterpret_cast<const uint4v*>(kb + int64_t(r.r[i]) * stride);
+        const uint4v* src = reinterpret_cast<const uint4v*>(kb + int64_t(r.r) * stride);
+        kreg[0] = src[0];
+        kreg[1] = src[8];
     };
     auto load_v = [&](uint32_t it, const TileRows& r) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
-#pragma unroll
-        for (int i = 0; i < kStageSteps; i++)
-            vreg[i] = *reinterpret_cast<const uint4v*>(vb + int64_t(r.r[i]) * stride);
+        const uint4v* src = reinterpret_cast<const uint4v*>(vb + int64_t(r.r) * stride);
+        vreg[0] = src[0];
+        vreg[1] = src[8];
     };
     auto store_k = [&](uint32_t buf) {
-        uint16_t* sk = s_k0 + buf * kKTileHalves + k_st;
-#pragma unroll
-        for (int i = 0; i < kStageSteps; i++)
-            *reinterpret_cast<uint4v*>(sk + kStageRows * i * kKPitch) = kreg[i];
+        uint4v* dst = reinterpret_cast<uint4v*>(s_k0 + buf * kKTileHalves + k_st);
+        dst[0] = kreg[0];
+        dst[8] = kreg[1];
     };
     auto store_v = [&](uint32_t buf) {
-        uint16_t* sv = s_v0 + buf * kVTileHalves + v_st;
-#pragma unroll
-        for (int i = 0; i < kStageSteps; i++)
-            *reinterpret_cast<uint4v*>(sv + kStageRows * i * kVPitch) = vreg[i];
+        uint16_t* sv = s_v0 + buf * kVTileHalves;
+        *reinterpret_cast<uint4v*>(sv + v_st) = vreg[0];
+        *reinterpret_cast<uint4v*>(sv + v_st2) = vreg[1];
     };
 
     // ---- V^T operand reads.  16-lane group q = lane / 16, lane i = 4k + r inside it:
@@ -333,7 +348,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     };
     // Given the lane's maximum over a sub-tile's scores: the row maximum and, when a row
     // outgrows the reference maximum, the rescale of m_ref, l and O.
-    auto finish_max = [&](float mraw) {
+    // `pending` are probabilities that were taken relative to the old reference and have not
+    // been multiplied into O yet (the pipeline below keeps one sub-tile of them).
+    auto finish_max = [&](float mraw, half8 (*pending)[2]) {
         const LanePair both = half_wave_pair(mraw);
         const float m_tile = fmaxf(both.lo, both.hi) * p.scale_log2;
         if (__any(m_tile > m_ref + kRescaleSlack)) {
@@ -341,6 +358,13 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             const float alpha = fast_exp2(m_ref - m_new);
             m_ref = m_new;
             l_run *= alpha;
+            if (pending) {
+                const _Float16 ah = static_cast<_Float16>(alpha);
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) (*pending)[u][j] *= ah;
+            }
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
@@ -352,7 +376,14 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         float mraw = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
-        finish_max(mraw);
+        finish_max(mraw, nullptr);
+    };
+    auto mask_and_max_pending = [&](const TileInfo& ti, int sub, float16v& sacc, half8 (&pending)[2]) {
+        apply_mask(ti, sub, sacc);
+        float mraw = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
+        finish_max(mraw, &pending);
     };
     // P^T = exp2(S^T * scale - m_ref) of a sub-tile as B operands of the second product;
     // adds to l.
@@ -397,18 +428,38 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
     };
 
-    // One pipeline phase with the two instruction streams interleaved by hand: the 8
-    // MFMAs of the scores of sub-tile (it_q, sub_q), each followed by a slice of the softmax
-    // arithmetic of the previous sub-tile (scores s_in), then the 8 MFMAs of the second
-    // product for (it_v, sub_v).  On this part a 32x32x16 MFMA keeps the vector ALU to
-    // itself for only half of its 32 cycles and transcendentals run beside it, so vector
-    // work placed between MFMAs is nearly free, while vector work after a burst of MFMAs
-    // is not; the scheduling barriers keep the compiler from regrouping the slices.
-    // Operands are fetched from LDS two steps ahead.
+#ifdef GHIP_EXP_TIMELINE
+    uint32_t tl_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint32_t tl_last = uint32_t(__builtin_readcyclecounter());
+#define TL_MARK(slot)                                                   \
+    do {                                                                \
+        const uint32_t now_ = uint32_t(__builtin_readcyclecounter());   \
+        tl_acc[slot] += now_ - tl_last;                                 \
+        tl_last = now_;                                                 \
+    } while (0)
+#else
+#define TL_MARK(slot) do {} while (0)
+#endif
+    int tl_base = 0;
+    (void)tl_base;
+    // One phase of the three-stage pipeline, instruction streams interleaved by hand.  For
+    // sub-tile j it runs
+    //   the 8 MFMAs of the scores of sub-tile j + 1        (K operands from LDS),
+    //   the softmax arithmetic of sub-tile j               (scores s_in -> probabilities p_out),
+    //   the 8 MFMAs of the second product of sub-tile j - 1 (V^T operands from LDS, p_prev),
+    // with one score element turned into a probability after every MFMA, so that all 16
+    // MFMAs of a phase have vector work of an *earlier* sub-tile to hide: on this part a
+    // 32x32x16 MFMA keeps the vector ALU to itself for only half of its 32 cycles and
+    // transcendentals run beside it, so a few vector instructions between MFMAs are free
+    // while the same instructions after a burst of MFMAs are not.  The scheduling barriers
+    // and the empty asm statements keep the compiler from regrouping or sinking the slices.
+    // Operands are fetched from LDS two steps ahead.  Step e scales element e + 1, takes the
+    // exponential of element e and sums / packs element e - 1.
     auto fused_phase = [&](const TileInfo& ti_q, uint32_t kbuf, int sub_q, float16v& s_out,
-                           const float16v& s_in, uint32_t it_v /* V buffer */, int sub_v) {
+                           const float16v& s_in, half8 (&p_out)[2], uint32_t vbuf, int sub_v,
+                           const half8 (&p_prev)[2]) {
         const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
-        const uint16_t* sv = s_v0 + it_v * kVTileHalves + 32 * sub_v * kVPitch;
+        const uint16_t* sv = s_v0 + vbuf * kVTileHalves + 32 * sub_v * kVPitch;
         auto k_operand = [&](int s8) -> uint4v {
             return *reinterpret_cast<const uint4v*>(krow + 16 * s8);
         };
@@ -422,81 +473,61 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
                             (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch)));
             return uint4v{lo.x, lo.y, hi.x, hi.y};
         };
-#ifdef GHIP_EXP_RING4
-        constexpr int kRing = 4;
-#else
         constexpr int kRing = 3;
-#endif
         uint4v ring[kRing];
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(i);
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        float psum = 0.0f;
+        float psum = 0.0f, mraw = -INFINITY;
+        float pe[16];
         uint32_t pw[8];
-        // The softmax slices are themselves pipelined over the steps, so that no step
-        // waits on its own results: step s8 scales the scores of slice s8 + 1, takes the
-        // exponentials of slice s8 and sums and packs slice s8 - 1.
-        float t0 = __builtin_fmaf(s_in[0], p.scale_log2, -m_ref);
-        float t1 = __builtin_fmaf(s_in[1], p.scale_log2, -m_ref);
-        float ep0 = 0.0f, ep1 = 0.0f;
+        float tn = __builtin_fmaf(s_in[0], p.scale_log2, -m_ref);
+        // the vector work of step e (0..15); element e - 1 is finished here, in pairs
+        auto softmax_step = [&](int e) {
+            pe[e] = fast_exp2(tn);
+            if (e < 15) tn = __builtin_fmaf(s_in[e + 1], p.scale_log2, -m_ref);
+            if (e > 0) psum += pe[e - 1];
+            if (e > 0 && (e & 1) == 0) pw[e / 2 - 1] = pack_f16x2(pe[e - 2], pe[e - 1]);
+            asm volatile("" : "+v"(pe[e]), "+v"(tn), "+v"(psum));
+            if (e > 0 && (e & 1) == 0) asm volatile("" : "+v"(pw[e / 2 - 1]));
+        };
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++) {
-#ifdef GHIP_EXP_NO_QK
-            c[s8] += bq[s8][0];
-#else
             if (s8 + kRing - 1 < 8) ring[(s8 + kRing - 1) % kRing] = k_operand(s8 + kRing - 1);
             c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq[s8], c, 0, 0, 0);
-#endif
             if constexpr (kQF32)
                 c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq_lo[s8], c, 0, 0, 0);
-            const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
-            if (s8 < 7) {
-                t0 = __builtin_fmaf(s_in[2 * s8 + 2], p.scale_log2, -m_ref);
-                t1 = __builtin_fmaf(s_in[2 * s8 + 3], p.scale_log2, -m_ref);
-            }
-            if (s8 > 0) {
-                psum += ep0;
-                psum += ep1;
-                pw[s8 - 1] = pack_f16x2(ep0, ep1);
-            }
-            ep0 = e0;
-            ep1 = e1;
-            // pin the slice here: without it the optimiser sinks the softmax arithmetic
-            // below the (rarely taken) mask branch, away from the MFMAs it should hide behind
-            asm volatile("" : "+v"(ep0), "+v"(ep1), "+v"(t0), "+v"(t1), "+v"(psum));
-            if (s8 > 0) asm volatile("" : "+v"(pw[s8 - 1]));
+            softmax_step(s8);
             __builtin_amdgcn_sched_barrier(0);
         }
-        psum += ep0;
-        psum += ep1;
-        pw[7] = pack_f16x2(ep0, ep1);
-        l_run += psum;
-        const half8 bp0 = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
-        const half8 bp1 = as_half8(uint4v{pw[4], pw[5], pw[6], pw[7]});
+        TL_MARK(tl_base + 1);
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = v_operand(i);
         apply_mask(ti_q, sub_q, c);  // rare; the maximum of the new scores rides along below
-        float mraw = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            mraw = fmaxf(fmaxf(mraw, c[2 * i]), c[2 * i + 1]);
-#ifdef GHIP_EXP_NO_PV
-            oacc[i & 3][i] += float(((i >> 2) ? bp1 : bp0)[0]);
-#else
             if (i + kRing - 1 < 8) ring[(i + kRing - 1) % kRing] = v_operand(i + kRing - 1);
             oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % kRing]),
-                                                                 (i >> 2) ? bp1 : bp0, oacc[i & 3], 0, 0, 0);
-#endif
+                                                                 p_prev[i >> 2], oacc[i & 3], 0, 0, 0);
+            softmax_step(8 + i);
+            mraw = fmaxf(fmaxf(mraw, c[2 * i]), c[2 * i + 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        TL_MARK(tl_base + 2);
+        psum += pe[15];
+        pw[7] = pack_f16x2(pe[14], pe[15]);
+        l_run += psum;
+        p_out[0] = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
+        p_out[1] = as_half8(uint4v{pw[4], pw[5], pw[6], pw[7]});
         s_out = c;
-        finish_max(mraw);
+        finish_max(mraw, &p_out);
+        TL_MARK(tl_base + 3);
     };
 
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
     // ---- prologue.  In LDS: K of the first two tiles, V of the first.  In flight: K of the
     // third tile, V of the second.  Row lookups: one tile further.
-    // K of tile t_begin + j lives in buffer j % 3, V in buffer j & 1.
+    // K and V of tile t_begin + j live in buffers j % 3.
     TileRows rows_v, rows_k;  // rows of the tiles whose V / K is loaded next
     tile_rows(t_begin, rows_k);
     load_k(t_begin, rows_k);
@@ -513,14 +544,14 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     tile_rows(t_begin + 3, rows_k);
     __syncthreads();
 
-    // The loop is software pipelined over 32-key sub-tiles: while the vector ALU turns
-    // the scores of one sub-tile into probabilities, the matrix pipe already computes the
-    // scores of the next one, and the maximum of those is taken while the second product
-    // of the current sub-tile runs.  s0 holds the scores of sub-tile 0 of the current tile
-    // on entry to an iteration; K is therefore staged one tile ahead of V and kept in three
-    // buffers (the tile being finished, the next one, the one being written), which leaves
-    // one barrier per tile.
+    // The loop is software pipelined three deep over 32-key sub-tiles (see fused_phase).
+    // On entry to an iteration s0 holds the scores of sub-tile 0 of tile `it` and p_old the
+    // probabilities of sub-tile 1 of tile it - 1, whose second product is still due.  K is
+    // therefore staged one tile ahead of V, and both are kept in three buffers (K: the tile
+    // being finished, the next one, the one being written; V: the previous tile, the
+    // current one, the one being written), which leaves one barrier per tile.
     float16v s0, s1;
+    half8 p_old[2], p_new[2];
     {
         const TileInfo first = tile_info(t_begin);
         if (first.active) {
@@ -529,57 +560,78 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
     }
     uint32_t kb_cur = 0, kb_next = 1, kb_store = 2;  // K buffers of tiles it, it + 1, it + 2
-    uint32_t vb_cur = 0;                              // V buffer of tile it
+    uint32_t vb_prev = 2, vb_cur = 0, vb_store = 1;  // V buffers of tiles it - 1, it, it + 1
+    bool prev_active = false;                        // tile it - 1 was computed by this wave
     for (uint32_t it = t_begin; it < n_tiles; it++) {
-        // Unconditional staging (indices clamp at the last tile): loads inside a branch
-        // would force a full wait at the join.  Stores past the last tile go to buffers
-        // nobody reads any more.
-#ifndef GHIP_EXP_NO_LSTORE
-        store_k(kb_store);     // K of tile it + 2
-        store_v(vb_cur ^ 1);   // V of tile it + 1
-#endif
-#ifndef GHIP_EXP_NO_GLOAD
-        load_k(it + 3, rows_k);
-        load_v(it + 2, rows_v);
-#endif
-        rows_v = rows_k;
-#ifndef GHIP_EXP_NO_ROWS
-        tile_rows(it + 4, rows_k);
-#endif
-
         const TileInfo cur = tile_info(it);
         const TileInfo nxt = tile_info(it + 1);
-        half8 bp[2];
-        if (cur.active && nxt.active) {  // the common case
-            fused_phase(cur, kb_cur, 1, s1, s0, vb_cur, 0);
-            fused_phase(nxt, kb_next, 0, s0, s1, vb_cur, 1);
-        } else {
-            if (cur.active) fused_phase(cur, kb_cur, 1, s1, s0, vb_cur, 0);
-            if (nxt.active) scores(kb_next, 0, s0);
-            if (cur.active) {
-                probabilities(s1, bp);
-                accumulate(vb_cur, 1, bp);
-            }
-            if (nxt.active) mask_and_max(nxt, 0, s0);
+        const bool fused = prev_active && cur.active && nxt.active;  // the common case
+        TL_MARK(0);
+        if (fused) {
+            tl_base = 0;
+            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old);
         }
+        // Staging, unconditional (indices clamp at the last tile): loads inside a branch would
+        // force a full wait at the join; stores past the last tile go to buffers nobody reads
+        // any more.  It sits between the two phases: the loads issued an iteration ago have
+        // had a phase more to arrive, and the target buffers (K of tile it - 1, V of tile
+        // it - 2) have been free since the last barrier.
+        store_k(kb_store);  // K of tile it + 2
+        store_v(vb_store);  // V of tile it + 1
+        load_k(it + 3, rows_k);
+        load_v(it + 2, rows_v);
+        rows_v = rows_k;
+        tile_rows(it + 4, rows_k);
+        TL_MARK(7);
+        if (fused) {
+            tl_base = 3;
+            fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new);
+        } else {
+            // the same three stages one after the other, each only where it applies
+            if (prev_active) accumulate(vb_prev, 1, p_old);
+            if (cur.active) {
+                scores(kb_cur, 1, s1);
+                probabilities(s0, p_new);
+                mask_and_max_pending(cur, 1, s1, p_new);
+                accumulate(vb_cur, 0, p_new);
+                probabilities(s1, p_old);
+            }
+            if (nxt.active) {
+                scores(kb_next, 0, s0);
+                mask_and_max_pending(nxt, 0, s0, p_old);
+            }
+        }
+        prev_active = cur.active;
         __syncthreads();
-        const uint32_t freed = kb_cur;
+        TL_MARK(0);
+        const uint32_t kfreed = kb_cur;
         kb_cur = kb_next;
         kb_next = kb_store;
-        kb_store = freed;
-        vb_cur ^= 1;
+        kb_store = kfreed;
+        const uint32_t vfreed = vb_prev;
+        vb_prev = vb_cur;
+        vb_cur = vb_store;
+        vb_store = vfreed;
     }
+    if (prev_active) accumulate(vb_prev, 1, p_old);  // drain: sub-tile 1 of the last tile
     }
 
+#ifdef GHIP_EXP_TIMELINE
+    if (p.lse && lane == 0) {
+        float* tl = p.lse + size_t(blockIdx.x) * 64 + wave * 8;
+        for (int i = 0; i < 8; i++) tl[i] = float(tl_acc[i]);
+    }
+    if (true) return;
+#endif
     if (!wave_active) return;
     {
         const LanePair both = half_wave_pair(l_run);
         l_run = both.lo + both.hi;
     }
     if (q_row >= p.seq_q) return;
-    if (gridDim.z > 1) {
+    if (p.n_splits > 1) {
         // partial result of this key range: O unnormalised, (m_ref, l) beside it
-        const size_t row = (size_t(blockIdx.z) * p.num_heads + head) * p.seq_q + q_row;
+        const size_t row = (size_t(split) * p.num_heads + head) * p.seq_q + q_row;
         float* po = p.part_o + row * kHeadDim;
 #pragma unroll
         for (int t = 0; t < 4; t++)
@@ -828,7 +880,10 @@ int launch_attention(const granite_hip_attention_args& a) {
             p.final_head_stride = a.out_head_stride;
         }
     }
-    dim3 grid(q_tiles, a.num_heads, n_splits);
+    p.q_tiles = q_tiles;
+    p.n_splits = n_splits;
+    if (uint64_t(q_tiles) * a.num_heads * n_splits > 0x7FFFFFFFull) return GRANITE_HIP_EINVAL;
+    dim3 grid(q_tiles * a.num_heads * n_splits);
     const int rows = !a.block_table ? kRowsContiguous
                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
