@@ -237,7 +237,8 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     struct TileRows {
         uint32_t r;  // row of key ld_r
     };
-    uint4v kreg[2], vreg[2];
+    // two register sets: the loads of an iteration are stored two iterations later
+    uint4v kreg_a[2], vreg_a[2], kreg_b[2], vreg_b[2];
 
     auto tile_rows = [&](uint32_t it, TileRows& r) {
         it = min(it, n_tiles - 1);
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         r.r = key_row<kRows>(p, min(key0 + ld_r, last), seg_b);
     };
     // K and V of a tile are moved separately: K runs one tile ahead of V (see the loop).
-    auto load_k = [&](uint32_t it, const TileRows& r) {
+    auto load_k = [&](uint32_t it, const TileRows& r, uint4v (&kreg)[2]) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
@@ -256,7 +257,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         kreg[0] = src[0];
         kreg[1] = src[8];
     };
-    auto load_v = [&](uint32_t it, const TileRows& r) {
+    auto load_v = [&](uint32_t it, const TileRows& r, uint4v (&vreg)[2]) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
@@ -265,12 +266,12 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         vreg[0] = src[0];
         vreg[1] = src[8];
     };
-    auto store_k = [&](uint32_t buf) {
+    auto store_k = [&](uint32_t buf, const uint4v (&kreg)[2]) {
         uint4v* dst = reinterpret_cast<uint4v*>(s_k0 + buf * kKTileHalves + k_st);
         dst[0] = kreg[0];
         dst[8] = kreg[1];
     };
-    auto store_v = [&](uint32_t buf) {
+    auto store_v = [&](uint32_t buf, const uint4v (&vreg)[2]) {
         uint16_t* sv = s_v0 + buf * kVTileHalves;
         *reinterpret_cast<uint4v*>(sv + v_st) = vreg[0];
         *reinterpret_cast<uint4v*>(sv + v_st2) = vreg[1];
@@ -526,22 +527,25 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
 
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
     // ---- prologue.  In LDS: K of the first two tiles, V of the first.  In flight: K of the
-    // third tile, V of the second.  Row lookups: one tile further.
+    // third and fourth tile, V of the second and third.  Row lookups: one tile further.
     // K and V of tile t_begin + j live in buffers j % 3.
     TileRows rows_v, rows_k;  // rows of the tiles whose V / K is loaded next
     tile_rows(t_begin, rows_k);
-    load_k(t_begin, rows_k);
-    load_v(t_begin, rows_k);
+    load_k(t_begin, rows_k, kreg_a);
+    load_v(t_begin, rows_k, vreg_a);
     tile_rows(t_begin + 1, rows_v);
-    store_k(0);
-    store_v(0);
-    load_k(t_begin + 1, rows_v);
+    load_k(t_begin + 1, rows_v, kreg_b);
     tile_rows(t_begin + 2, rows_k);
-    store_k(1);
-    load_v(t_begin + 1, rows_v);
-    load_k(t_begin + 2, rows_k);
-    rows_v = rows_k;
-    tile_rows(t_begin + 3, rows_k);
+    store_k(0, kreg_a);
+    store_v(0, vreg_a);
+    store_k(1, kreg_b);
+    // set a: K of tile t_begin + 2, V of t_begin + 1; set b: K of t_begin + 3, V of t_begin + 2
+    load_k(t_begin + 2, rows_k, kreg_a);
+    load_v(t_begin + 1, rows_v, vreg_a);
+    tile_rows(t_begin + 3, rows_v);
+    load_v(t_begin + 2, rows_k, vreg_b);
+    load_k(t_begin + 3, rows_v, kreg_b);
+    tile_rows(t_begin + 4, rows_k);  // rows_v now belongs to tile t_begin + 3, rows_k to + 4
     __syncthreads();
 
     // The loop is software pipelined three deep over 32-key sub-tiles (see fused_phase).
@@ -562,7 +566,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     uint32_t kb_cur = 0, kb_next = 1, kb_store = 2;  // K buffers of tiles it, it + 1, it + 2
     uint32_t vb_prev = 2, vb_cur = 0, vb_store = 1;  // V buffers of tiles it - 1, it, it + 1
     bool prev_active = false;                        // tile it - 1 was computed by this wave
-    for (uint32_t it = t_begin; it < n_tiles; it++) {
+    auto iteration = [&](uint32_t it, uint4v (&kreg)[2], uint4v (&vreg)[2]) {
         const TileInfo cur = tile_info(it);
         const TileInfo nxt = tile_info(it + 1);
         const bool fused = prev_active && cur.active && nxt.active;  // the common case
@@ -573,15 +577,15 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         // Staging, unconditional (indices clamp at the last tile): loads inside a branch would
         // force a full wait at the join; stores past the last tile go to buffers nobody reads
-        // any more.  It sits between the two phases: the loads issued an iteration ago have
-        // had a phase more to arrive, and the target buffers (K of tile it - 1, V of tile
-        // it - 2) have been free since the last barrier.
-        store_k(kb_store);  // K of tile it + 2
-        store_v(vb_store);  // V of tile it + 1
-        load_k(it + 3, rows_k);
-        load_v(it + 2, rows_v);
+        // any more.  It sits between the two phases; what is stored now was requested two
+        // iterations ago (the register set alternates), and the target buffers (K of tile
+        // it - 1, V of tile it - 2) have been free since the last barrier.
+        store_k(kb_store, kreg);  // K of tile it + 2
+        store_v(vb_store, vreg);  // V of tile it + 1
+        load_k(it + 4, rows_k, kreg);
+        load_v(it + 3, rows_v, vreg);
         rows_v = rows_k;
-        tile_rows(it + 4, rows_k);
+        tile_rows(it + 5, rows_k);
         TL_MARK(7);
         if (fused) {
             tl_base = 3;
@@ -612,6 +616,11 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         vb_prev = vb_cur;
         vb_cur = vb_store;
         vb_store = vfreed;
+    };
+    for (uint32_t it = t_begin; it < n_tiles; it += 2) {
+        iteration(it, kreg_a, vreg_a);
+        if (it + 1 >= n_tiles) break;
+        iteration(it + 1, kreg_b, vreg_b);
     }
     if (prev_active) accumulate(vb_prev, 1, p_old);  // drain: sub-tile 1 of the last tile
     }
