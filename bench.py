@@ -39,14 +39,15 @@ for p in (ROOT, ROOT / "tests"):
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (see profiles/); None until measured.
-CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
-
+# HBM bytes per launch of each workload's dominant kernel, from two
+# `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE), each scaled
+# by what the same counter reads for the identity gather of
+# `--workload copy_calibration` (1.998 KiB per FETCH_SIZE unit, 1.000 KiB per
+# WRITE_SIZE unit); the summaries are under profiles/.
 MEASURED_TRAFFIC = {
-    "paged_decode": None,
-    "prefill": None,
-    "chunked_prefill": None,
+    "paged_decode": 1134673288,    # decode_stream_kernel; algorithmic 1132236296
+    "prefill": 42546817,           # attention_tiles_kernel; algorithmic 41943040
+    "chunked_prefill": 179564192,  # attention_tiles_kernel; algorithmic 153092096
 }
 
 

@@ -10,46 +10,60 @@
 // (fp32 scores and softmax, no epsilon, key k visible iff k <= start_pos + q;
 // tree: cache keys visible, tree key j visible iff j is q or an ancestor).
 //
-// Structure.  grid = (query tiles of 256 rows, query heads, key splits); 8 waves,
-// each owning 32 query rows (one workgroup per CU, two waves per SIMD: a K/V
-// tile staged in LDS serves 256 query rows).  Keys are walked in tiles of 64.  Per tile every wave
-// computes, with v_mfma_f32_32x32x16_f16,
+// Structure.  One workgroup of 8 waves (two per SIMD) per (query tile of 256
+// rows, query head, key split); a wave owns 32 query rows, and a K/V tile
+// staged in LDS serves all 256.  Workgroup ids are remapped so that the
+// workgroups that stream the same K/V range (same KV head, same split) land on
+// the same XCD and share its L2.  Keys are walked in tiles of 64, each handled
+// as two 32-key sub-tiles.  Per sub-tile every wave computes, with
+// v_mfma_f32_32x32x16_f16,
 //
 //   S^T[key, q]  = K[key, :] . Q[q, :]          (A = K from LDS, B = Q in VGPRs)
-//   softmax in the result layout: a lane owns one query row and 32 of the 64
-//   keys, so max/sum are in-lane plus one cross-half shuffle
+//   softmax in the result layout: a lane owns one query row and 16 of the 32
+//   keys, so max/sum are in-lane plus one exchange between the wave's halves
 //   O^T[d, q]   += V^T[d, key] . P^T[key, q]    (A = V^T from LDS, B = P in VGPRs)
 //
 // Computing the transposed products makes the softmax output of the first
-// MFMA land exactly in the B-operand layout of the second once the keys of
-// each 16-key step are taken in the order described next.
+// MFMA land exactly in the B-operand layout of the second: with the keys of a
+// tile in their natural order the lane that owns S^T rows (keys) 8a + 4g + b
+// needs, as B operand of the second MFMA, k-index 8g + 4a' + b for key
+// 16u + 8a' + 4g + b, and the A operand (V^T) simply reads its keys in that
+// order.
 //
-// With the keys of a tile in their natural order the lane that owns S^T rows
-// (keys) 8a + 4g + b needs, as B operand of the second MFMA, k-index
-// 8g + 4a' + b for key 16u + 8a' + 4g + b: the A operand (V^T) simply reads
-// its keys in that order.
+// Pipeline.  The three stages of consecutive sub-tiles run in one phase
+// (fused_phase): the MFMAs of the scores of sub-tile j + 1, the softmax
+// arithmetic of sub-tile j and the MFMAs of the second product of sub-tile
+// j - 1, with one score element turned into a probability after every MFMA.
+// On this part a 32x32x16 MFMA keeps the vector ALU busy for only half of its
+// 32 cycles and transcendentals run beside it, so vector work placed between
+// MFMAs costs next to nothing while the same work after a burst of MFMAs costs
+// its full time.
 //
-// Data movement.  K/V tiles go global -> registers -> LDS, two LDS buffers,
-// one barrier per tile: while tile i is being multiplied, tile i+1 is written
-// to the other buffer, tile i+2 is in flight from HBM and the block-table rows
-// of tile i+3 are being fetched.  Both tiles are stored row-major as they lie
-// in memory (a thread moves the same four rows of K and of V, so one row
-// lookup serves both).  K rows have a pitch of 136 halves.  V rows have no
-// padding; the four 64-byte chunks of a row are XOR-swizzled with the low two
-// bits of the key instead.  The V^T operand comes out of the row-major tile
-// through ds_read_b64_tr_b16: inside a 16-lane group, lane 4k + r supplies the
-// address of four consecutive head-dim elements of key k and lane j receives
-// element j & 3 of the four lanes {4k' + (j >> 2)}, i.e. one head-dim element
-// of four consecutive keys.  With the swizzle the four key rows a group reads
-// fall into different bank groups, so neither the 16-byte stores nor the
-// transposing reads conflict.  The head-dim order of the A-operand rows is
-// chosen so that each lane ends up with runs of 8 consecutive output elements.
+// Data movement.  K/V tiles go global -> registers -> LDS; a thread moves two
+// 16-byte pieces of one key row of K and of V (one row lookup per thread and
+// tile).  What is loaded in one iteration is stored two iterations later (two
+// register sets), between the two phases of an iteration; row lookups run one
+// tile further ahead.  K is needed a tile earlier than V, so LDS holds three K
+// tiles (being finished, next, being written) and three V tiles (previous,
+// current, being written), which leaves one barrier per tile.  Both are stored
+// row-major as they lie in memory.  K rows have a pitch of 136 halves.  V rows
+// have no padding; the four 64-byte chunks of a row are XOR-swizzled with the
+// low two bits of the key instead.  The V^T operand comes out of the row-major
+// tile through ds_read_b64_tr_b16: inside a 16-lane group, lane 4k + r supplies
+// the address of four consecutive head-dim elements of key k and lane j
+// receives element j & 3 of the four lanes {4k' + (j >> 2)}, i.e. one head-dim
+// element of four consecutive keys.  With the swizzle the four key rows a
+// group reads fall into different bank groups, so neither the 16-byte stores
+// nor the transposing reads conflict.  The head-dim order of the A-operand
+// rows is chosen so that each lane ends up with runs of 8 consecutive output
+// elements.
 //
 // Softmax rescaling is lazy: probabilities are taken relative to a per-row
 // reference maximum that is only moved (and O, l rescaled) when the row
-// maximum of a tile exceeds it by more than 2^8.  Results are identical up to
-// rounding, P stays inside half range, and the accumulators are left alone in
-// almost every tile.
+// maximum of a sub-tile exceeds it by more than 2^8 (the probabilities of the
+// sub-tile still waiting for its second product are rescaled with them).
+// Results are identical up to rounding, P stays inside half range, and the
+// accumulators are left alone in almost every tile.
 //
 // Algorithmic work: 4 * D flops per visible (query, key) pair.
 #include <cstdlib>
@@ -429,20 +443,6 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
     };
 
-#ifdef GHIP_EXP_TIMELINE
-    uint32_t tl_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    uint32_t tl_last = uint32_t(__builtin_readcyclecounter());
-#define TL_MARK(slot)                                                   \
-    do {                                                                \
-        const uint32_t now_ = uint32_t(__builtin_readcyclecounter());   \
-        tl_acc[slot] += now_ - tl_last;                                 \
-        tl_last = now_;                                                 \
-    } while (0)
-#else
-#define TL_MARK(slot) do {} while (0)
-#endif
-    int tl_base = 0;
-    (void)tl_base;
     // One phase of the three-stage pipeline, instruction streams interleaved by hand.  For
     // sub-tile j it runs
     //   the 8 MFMAs of the scores of sub-tile j + 1        (K operands from LDS),
@@ -501,7 +501,6 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             softmax_step(s8);
             __builtin_amdgcn_sched_barrier(0);
         }
-        TL_MARK(tl_base + 1);
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = v_operand(i);
         apply_mask(ti_q, sub_q, c);  // rare; the maximum of the new scores rides along below
@@ -514,7 +513,6 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             mraw = fmaxf(fmaxf(mraw, c[2 * i]), c[2 * i + 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        TL_MARK(tl_base + 2);
         psum += pe[15];
         pw[7] = pack_f16x2(pe[14], pe[15]);
         l_run += psum;
@@ -522,7 +520,6 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         p_out[1] = as_half8(uint4v{pw[4], pw[5], pw[6], pw[7]});
         s_out = c;
         finish_max(mraw, &p_out);
-        TL_MARK(tl_base + 3);
     };
 
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
@@ -570,9 +567,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const TileInfo cur = tile_info(it);
         const TileInfo nxt = tile_info(it + 1);
         const bool fused = prev_active && cur.active && nxt.active;  // the common case
-        TL_MARK(0);
         if (fused) {
-            tl_base = 0;
             fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old);
         }
         // Staging, unconditional (indices clamp at the last tile): loads inside a branch would
@@ -586,9 +581,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         load_v(it + 3, rows_v, vreg);
         rows_v = rows_k;
         tile_rows(it + 5, rows_k);
-        TL_MARK(7);
         if (fused) {
-            tl_base = 3;
             fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new);
         } else {
             // the same three stages one after the other, each only where it applies
@@ -607,7 +600,6 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         prev_active = cur.active;
         __syncthreads();
-        TL_MARK(0);
         const uint32_t kfreed = kb_cur;
         kb_cur = kb_next;
         kb_next = kb_store;
@@ -625,13 +617,6 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     if (prev_active) accumulate(vb_prev, 1, p_old);  // drain: sub-tile 1 of the last tile
     }
 
-#ifdef GHIP_EXP_TIMELINE
-    if (p.lse && lane == 0) {
-        float* tl = p.lse + size_t(blockIdx.x) * 64 + wave * 8;
-        for (int i = 0; i < 8; i++) tl[i] = float(tl_acc[i]);
-    }
-    if (true) return;
-#endif
     if (!wave_active) return;
     {
         const LanePair both = half_wave_pair(l_run);
