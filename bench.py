@@ -39,6 +39,8 @@ for p in (ROOT, ROOT / "tests"):
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
+CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
+
 # HBM bytes per launch of each workload's dominant kernel, from two
 # `rocprofv3 --pmc` runs of this file (FETCH_SIZE, then WRITE_SIZE), each scaled
 # by what the same counter reads for the identity gather of
@@ -427,7 +429,8 @@ def main() -> int:
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": head["unit"] != "us", "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": head["workload"], "device": info.name.decode(), "arch": info.arch.decode(),
+        "config": {"workload": head["workload"], "device": info.name.decode() or info.arch.decode(),
+                   "arch": info.arch.decode(),
                    "compute_units": info.compute_units},
     }
     if "roofline" in head:
