@@ -123,22 +123,44 @@ __device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(
 
 // Row of the K/V array that holds key `idx`: of the cache segment (through the
 // block table when paged) or, with `extra`, of the extra segment (row = idx).
-// Branch-free on purpose: a load inside a conditional makes the compiler wait
-// for every outstanding load at the join, which would serialise the pipeline.
+// In two steps, so that the table entry can stay in flight while other loads are
+// issued: row_lookup() issues the table load and keeps the offset inside the
+// block; row_finish() combines them where the row is needed.  Branch-free on
+// purpose: a load inside a conditional makes the compiler wait for every
+// outstanding load at the join, which would serialise the pipeline.
+struct RowLookup {
+    uint32_t entry;  // block table entry (paged cache segment)
+    uint32_t add;    // offset inside the block, or the row itself where no table applies
+};
+
 template <int kRows>
-__device__ __forceinline__ uint32_t key_row(const AttnParams& p, uint32_t idx, bool extra) {
+__device__ __forceinline__ RowLookup row_lookup(const AttnParams& p, uint32_t idx, bool extra) {
+    RowLookup r;
     if constexpr (kRows == kRowsContiguous) {
-        return idx;
+        r.entry = 0;
+        r.add = idx;
     } else {
         const uint32_t t = extra ? 0u : idx;  // always a valid table position
-        uint32_t row;
         if constexpr (kRows == kRowsPagedPow2) {
-            row = (uint32_t(p.table[t >> p.bs_shift]) << p.bs_shift) + (t & (p.block_size - 1));
+            r.entry = uint32_t(p.table[t >> p.bs_shift]);
+            r.add = extra ? idx : (t & (p.block_size - 1));
         } else {
             const uint32_t blk = t / p.block_size;
-            row = uint32_t(p.table[blk]) * p.block_size + (t - blk * p.block_size);
+            r.entry = uint32_t(p.table[blk]);
+            r.add = extra ? idx : (t - blk * p.block_size);
         }
-        return extra ? idx : row;
+    }
+    return r;
+}
+
+template <int kRows>
+__device__ __forceinline__ uint32_t row_finish(const AttnParams& p, const RowLookup& r, bool extra) {
+    if constexpr (kRows == kRowsContiguous) {
+        return r.add;
+    } else {
+        const uint32_t e = extra ? 0u : r.entry;
+        if constexpr (kRows == kRowsPagedPow2) return (e << p.bs_shift) + r.add;
+        return e * p.block_size + r.add;
     }
 }
 
@@ -248,35 +270,36 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     const uint32_t v_st2 = ld_r * kVPitch + (((((ld_c >> 2) + 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
     const uint32_t k_st = ld_r * kKPitch + 8 * ld_c;
 
-    struct TileRows {
-        uint32_t r;  // row of key ld_r
-    };
     // two register sets: the loads of an iteration are stored two iterations later
     uint4v kreg_a[2], vreg_a[2], kreg_b[2], vreg_b[2];
 
-    auto tile_rows = [&](uint32_t it, TileRows& r) {
+    // row of key ld_r of tile `it`: the lookup, and the row once the lookup has arrived
+    auto tile_lookup = [&](uint32_t it) -> RowLookup {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint32_t key0 = (seg_b ? it - tiles_a : it) * kBN;
         const uint32_t last = (seg_b ? len_b : len_a) - 1;
-        r.r = key_row<kRows>(p, min(key0 + ld_r, last), seg_b);
+        return row_lookup<kRows>(p, min(key0 + ld_r, last), seg_b);
+    };
+    auto tile_row = [&](uint32_t it, const RowLookup& r) -> uint32_t {
+        return row_finish<kRows>(p, r, min(it, n_tiles - 1) >= tiles_a);
     };
     // K and V of a tile are moved separately: K runs one tile ahead of V (see the loop).
-    auto load_k = [&](uint32_t it, const TileRows& r, uint4v (&kreg)[2]) {
+    auto load_k = [&](uint32_t it, uint32_t row, uint4v (&kreg)[2]) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
-        const uint4v* src = reinterpret_cast<const uint4v*>(kb + int64_t(r.r) * stride);
+        const uint4v* src = reinterpret_cast<const uint4v*>(kb + int64_t(row) * stride);
         kreg[0] = src[0];
         kreg[1] = src[8];
     };
-    auto load_v = [&](uint32_t it, const TileRows& r, uint4v (&vreg)[2]) {
+    auto load_v = [&](uint32_t it, uint32_t row, uint4v (&vreg)[2]) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
-        const uint4v* src = reinterpret_cast<const uint4v*>(vb + int64_t(r.r) * stride);
+        const uint4v* src = reinterpret_cast<const uint4v*>(vb + int64_t(row) * stride);
         vreg[0] = src[0];
         vreg[1] = src[8];
     };
@@ -526,23 +549,35 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     // ---- prologue.  In LDS: K of the first two tiles, V of the first.  In flight: K of the
     // third and fourth tile, V of the second and third.  Row lookups: one tile further.
     // K and V of tile t_begin + j live in buffers j % 3.
-    TileRows rows_v, rows_k;  // rows of the tiles whose V / K is loaded next
-    tile_rows(t_begin, rows_k);
-    load_k(t_begin, rows_k, kreg_a);
-    load_v(t_begin, rows_k, vreg_a);
-    tile_rows(t_begin + 1, rows_v);
-    load_k(t_begin + 1, rows_v, kreg_b);
-    tile_rows(t_begin + 2, rows_k);
+    const uint32_t r0 = tile_row(t_begin, tile_lookup(t_begin));
+    const uint32_t r1 = tile_row(t_begin + 1, tile_lookup(t_begin + 1));
+    const uint32_t r2 = tile_row(t_begin + 2, tile_lookup(t_begin + 2));
+    uint32_t row_v = tile_row(t_begin + 3, tile_lookup(t_begin + 3));  // of the tile whose V is loaded next
+    load_k(t_begin, r0, kreg_a);
+    load_v(t_begin, r0, vreg_a);
+    load_k(t_begin + 1, r1, kreg_b);
     store_k(0, kreg_a);
     store_v(0, vreg_a);
     store_k(1, kreg_b);
+    // From here on a lookup is issued two iterations before the loads that use it, and kept
+    // with the register set (a / b) that those loads fill.  The counter of outstanding loads
+    // is in order: a load's address then depends on nothing younger than the loads that the
+    // stores of the same iteration wait for anyway, and the K/V loads of the previous
+    // iteration stay in flight.  The prologue issues its loads in the loop's order (K, V,
+    // lookup; set a, then set b) so that the waits the compiler derives for the loop's first
+    // pass are those of every other pass.
     // set a: K of tile t_begin + 2, V of t_begin + 1; set b: K of t_begin + 3, V of t_begin + 2
-    load_k(t_begin + 2, rows_k, kreg_a);
-    load_v(t_begin + 1, rows_v, vreg_a);
-    tile_rows(t_begin + 3, rows_v);
-    load_v(t_begin + 2, rows_k, vreg_b);
-    load_k(t_begin + 3, rows_v, kreg_b);
-    tile_rows(t_begin + 4, rows_k);  // rows_v now belongs to tile t_begin + 3, rows_k to + 4
+    __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move the lookups to the front)
+    load_k(t_begin + 2, r2, kreg_a);
+    load_v(t_begin + 1, r1, vreg_a);
+    __builtin_amdgcn_sched_barrier(0);
+    RowLookup look_a = tile_lookup(t_begin + 4);
+    __builtin_amdgcn_sched_barrier(0);
+    load_k(t_begin + 3, row_v, kreg_b);
+    load_v(t_begin + 2, r2, vreg_b);
+    __builtin_amdgcn_sched_barrier(0);
+    RowLookup look_b = tile_lookup(t_begin + 5);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
 
     // The loop is software pipelined three deep over 32-key sub-tiles (see fused_phase).
@@ -563,7 +598,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     uint32_t kb_cur = 0, kb_next = 1, kb_store = 2;  // K buffers of tiles it, it + 1, it + 2
     uint32_t vb_prev = 2, vb_cur = 0, vb_store = 1;  // V buffers of tiles it - 1, it, it + 1
     bool prev_active = false;                        // tile it - 1 was computed by this wave
-    auto iteration = [&](uint32_t it, uint4v (&kreg)[2], uint4v (&vreg)[2]) {
+    auto iteration = [&](uint32_t it, uint4v (&kreg)[2], uint4v (&vreg)[2], RowLookup& look) {
         const TileInfo cur = tile_info(it);
         const TileInfo nxt = tile_info(it + 1);
         const bool fused = prev_active && cur.active && nxt.active;  // the common case
@@ -577,10 +612,11 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         // it - 1, V of tile it - 2) have been free since the last barrier.
         store_k(kb_store, kreg);  // K of tile it + 2
         store_v(vb_store, vreg);  // V of tile it + 1
-        load_k(it + 4, rows_k, kreg);
-        load_v(it + 3, rows_v, vreg);
-        rows_v = rows_k;
-        tile_rows(it + 5, rows_k);
+        const uint32_t row_k = tile_row(it + 4, look);
+        load_k(it + 4, row_k, kreg);
+        load_v(it + 3, row_v, vreg);
+        row_v = row_k;
+        look = tile_lookup(it + 6);
         if (fused) {
             fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new);
         } else {
@@ -609,10 +645,12 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         vb_cur = vb_store;
         vb_store = vfreed;
     };
+    // Always in pairs: past the last tile an iteration only finishes what is pending and
+    // stages into buffers nobody reads.  (Leaving the loop between the two makes the
+    // compiler wait for the previous iteration's loads before every store.)
     for (uint32_t it = t_begin; it < n_tiles; it += 2) {
-        iteration(it, kreg_a, vreg_a);
-        if (it + 1 >= n_tiles) break;
-        iteration(it + 1, kreg_b, vreg_b);
+        iteration(it, kreg_a, vreg_a, look_a);
+        iteration(it + 1, kreg_b, vreg_b, look_b);
     }
     if (prev_active) accumulate(vb_prev, 1, p_old);  // drain: sub-tile 1 of the last tile
     }
