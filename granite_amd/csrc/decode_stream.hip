@@ -1,21 +1,32 @@
 // Persistent ("stream") form of the decode attention kernel.
 //
-// The context of every (sequence, KV head) is cut into 32-token tiles; all
-// tiles of the batch form one flat list, ordered (sequence, head, tile).  The
-// list is cut into equal contiguous ranges, one per wave, and the grid is one
-// workgroup per compute unit (one wave per SIMD), so every wave streams the same
-// number of K/V bytes and there is no per-chunk workgroup start-up.  (Two
-// workgroups per CU measured slower: the older one wins the memory pipeline and
-// the younger finishes 25 % later.)  A wave that crosses from one (sequence, head) to the next
-// writes a partial (m, l, O) for the part it covered; the merge kernel combines
-// the partials of a (sequence, head), whose positions follow from the same
-// arithmetic.
+// The context of every sequence is cut into 32-token tiles; all tiles of the
+// batch form one flat list that is cut into equal contiguous ranges, one per
+// worker, and the grid is one workgroup per compute unit (one wave per SIMD),
+// so every wave streams the same number of K/V bytes and there is no per-chunk
+// workgroup start-up.  (Two workgroups per CU measured slower: the older one
+// wins the memory pipeline and the younger finishes 25 % later.)
+//
+// Two shapes of the list:
+//   * rows ("kPair"), when the number of heads is a multiple of 8: the list is
+//     ordered (sequence, group of 8 heads, tile) and a worker is a workgroup.
+//     Its four waves walk the same tiles, each for two heads that it alternates
+//     between, so a workgroup reads whole token rows (all heads of a token are
+//     contiguous in the pool) at about the same time.  Which memory channels a
+//     workgroup loads then does not depend on how the sequence lengths fall:
+//     with one head per wave, a batch of mixed lengths ran 11 % slower than one
+//     of equal lengths, and the waves' run times spread by +-15 %.
+//   * flat, otherwise: the list is ordered (sequence, head, tile) and a worker
+//     is a wave.
+// A worker that crosses from one (sequence, head) to the next writes a partial
+// (m, l, O) for the part it covered; the merge kernel combines the partials of
+// a (sequence, head), whose positions follow from the same arithmetic.
 //
 // There is no separate planning launch: every workgroup scans the sequence
 // lengths into tile counts and their prefix sums itself, in LDS (a few hundred
 // nanoseconds for a batch of 64), and looks everything up there afterwards, so
 // that none of the bookkeeping ever waits on global memory.  Workgroup 0 also
-// stores the prefix sums and the per-wave share for the merge kernel.
+// stores the prefix sums and the per-worker share for the merge kernel.
 //
 // Inside a wave the pipeline is three tiles deep: the block-table rows of tile
 // i+2 and the K/V rows of tile i+1 are in flight while tile i goes through the
@@ -29,10 +40,12 @@
 namespace ghip {
 namespace {
 
-// One 32-token tile of one (sequence, virtual head).
+// One entry of the flat list: a 32-token tile of one (sequence, list head).  A list
+// head is a virtual head (kv_head * q_groups + q_group) or, in the rows shape, a group
+// of 8 consecutive virtual heads.
 struct Cursor {
     uint32_t b;    // sequence
-    uint32_t vh;   // virtual head = kv_head * q_groups + q_group
+    uint32_t vh;   // list head
     uint32_t t;    // tile inside the sequence
     uint32_t nt;   // tiles of sequence b
     uint32_t len;  // tokens of sequence b
@@ -43,16 +56,16 @@ __device__ __forceinline__ uint32_t seq_len_of(const DecodeParams& p, uint32_t b
     return min(len, p.max_tokens);
 }
 
-// Next tile in (sequence, head, tile) order; skips empty sequences.  `more`
+// Next tile in (sequence, list head, tile) order (`lists` list heads); skips empty sequences.  `more`
 // false leaves the cursor where it is (the caller re-reads the last tile
 // instead of running off the end, so no load ever sits inside a branch).
 // `lens` holds the token count of every sequence, in LDS.
-__device__ __forceinline__ void advance(const DecodeParams& p, const uint32_t* lens, Cursor& c,
-                                        bool more) {
+__device__ __forceinline__ void advance(const DecodeParams& p, const uint32_t* lens, uint32_t lists,
+                                        Cursor& c, bool more) {
     if (!more) return;
     if (++c.t < c.nt) return;
     c.t = 0;
-    if (++c.vh < p.num_kv_heads * p.q_groups) return;
+    if (++c.vh < lists) return;
     c.vh = 0;
     do {
         ++c.b;
@@ -62,20 +75,23 @@ __device__ __forceinline__ void advance(const DecodeParams& p, const uint32_t* l
     if (c.b >= p.batch) c.b = p.batch - 1;  // never dereferenced past the end
 }
 
+// Heads of one list entry in the rows shape: two per wave.
+constexpr uint32_t kPairHeads = 2 * kWavesPerWG;
+
 struct TileRegs {
     half8 ka[2][4];
     uint4v vr[8];
 };
 
-template <bool kQF32, int kRows>
-__global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(DecodeParams p) {
+template <bool kQF32, int kRows, bool kPair>
+__global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(DecodeParams p) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15;
     const uint32_t g = lane >> 4;
     // wave-uniform by construction; saying so keeps every cursor in scalar registers
-    const uint32_t worker =
-        uint32_t(__builtin_amdgcn_readfirstlane(int(blockIdx.x * kWavesPerWG + wave)));
+    const uint32_t worker = uint32_t(
+        __builtin_amdgcn_readfirstlane(int(kPair ? blockIdx.x : blockIdx.x * kWavesPerWG + wave)));
 
     // ---- tile counts and their prefix sums, in LDS
     extern __shared__ uint32_t s_dyn[];
@@ -118,36 +134,38 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
         if (threadIdx.x == 0) s_prefix[p.batch] = tiles_total;
         __syncthreads();
     }
-    const uint32_t total = tiles_total * vheads;
+    const uint32_t lists = kPair ? vheads / kPairHeads : vheads;  // list heads
+    const uint32_t total = tiles_total * lists;
     const uint32_t per = max((total + p.workers - 1) / p.workers, p.min_per);
     if (blockIdx.x == 0) {  // for the merge kernel
         for (uint32_t i = threadIdx.x; i <= p.batch; i += blockDim.x) p.plan[kPlanHeader + i] = s_prefix[i];
         if (threadIdx.x == 0) {
             p.plan[0] = per;
             p.plan[1] = total;
+            p.plan[2] = kPair ? kPairHeads : 1;
         }
     }
     auto prefix_u = [&](uint32_t i) -> uint32_t {  // wave-uniform index: stays in a scalar register
         return uint32_t(__builtin_amdgcn_readfirstlane(int(s_prefix[i])));
     };
 
-    // ---- this wave's range of the flat tile list
+    // ---- this worker's range of the flat tile list
     const uint32_t u0 = worker * per;
     if (u0 >= total) return;
     const uint32_t n_units = min(per, total - u0);
 
-    // locate u0: largest b with prefix[b] * vheads <= u0
+    // locate u0: largest b with prefix[b] * lists <= u0
     Cursor first;
     {
         uint32_t lo = 0, hi = p.batch;  // invariant: prefix[lo]*vheads <= u0 < prefix[hi]*vheads
         while (hi - lo > 1) {
             const uint32_t mid = (lo + hi) >> 1;
-            if (prefix_u(mid) * vheads <= u0) lo = mid; else hi = mid;
+            if (prefix_u(mid) * lists <= u0) lo = mid; else hi = mid;
         }
         first.b = lo;
         first.nt = prefix_u(lo + 1) - prefix_u(lo);
         first.len = uint32_t(__builtin_amdgcn_readfirstlane(int(s_len[lo])));
-        const uint32_t in_seq = u0 - prefix_u(lo) * vheads;
+        const uint32_t in_seq = u0 - prefix_u(lo) * lists;
         first.vh = in_seq / first.nt;
         first.t = in_seq - first.vh * first.nt;
     }
@@ -157,8 +175,13 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
             kRows != kRowsContiguous ? p.tables + size_t(c.b) * p.max_blocks : nullptr;
         return tile_row<kRows>(p, table, c.t * kTile, lane, c.len);
     };
-    auto issue = [&](TileRegs& r, uint32_t rows, const Cursor& c) {
-        const uint32_t kvh = c.vh / p.q_groups;
+    // Virtual head a cursor stands for: in the rows shape, the wave's first (side 0) or
+    // second (side 1) head of the cursor's group.
+    auto head_of = [&](const Cursor& c, uint32_t side) -> uint32_t {
+        return kPair ? c.vh * kPairHeads + 2 * wave + side : c.vh;
+    };
+    auto issue = [&](TileRegs& r, uint32_t rows, uint32_t vh) {
+        const uint32_t kvh = vh / p.q_groups;
         const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride + 8 * g;
         const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * n;
 #pragma unroll
@@ -176,14 +199,26 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
         }
     };
 
-    half8 bq[4];
-    half8 bq_lo[kQF32 ? 4 : 1];
-    auto load_q = [&](const Cursor& c) {
-        const uint32_t kvh = c.vh / p.q_groups, qg = c.vh % p.q_groups;
+    // Running state of one (sequence, virtual head): Q as B operands (with fp32 Q, an fp16
+    // head and an fp16 remainder), the maximum, the sum and O.
+    struct HeadState {
+        half8 bq[4];
+        half8 bq_lo[kQF32 ? 4 : 1];
+        float m_run, l_run;
+        float4v acc[8];
+    };
+    auto clear = [&](HeadState& h) {
+        h.m_run = kNegBig;
+        h.l_run = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; t++) h.acc[t] = float4v{0, 0, 0, 0};
+    };
+    auto load_q = [&](uint32_t b, uint32_t vh, HeadState& h) {
+        const uint32_t kvh = vh / p.q_groups, qg = vh % p.q_groups;
         const uint32_t q_in_group = qg * 16 + n;
         const bool q_valid = q_in_group < p.group;
         const uint32_t qh = kvh * p.group + (q_valid ? q_in_group : 0);
-        const size_t off = (size_t(c.b) * p.num_heads + qh) * kHeadDim + 8 * g;
+        const size_t off = (size_t(b) * p.num_heads + qh) * kHeadDim + 8 * g;
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             if constexpr (kQF32) {
@@ -195,36 +230,31 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     const float xv = q_valid ? x[i] : 0.0f;
-                    _Float16 h = static_cast<_Float16>(xv);
-                    hi[i] = h;
-                    lo[i] = static_cast<_Float16>(xv - static_cast<float>(h));
+                    _Float16 hv = static_cast<_Float16>(xv);
+                    hi[i] = hv;
+                    lo[i] = static_cast<_Float16>(xv - static_cast<float>(hv));
                 }
-                bq[s] = hi;
-                bq_lo[s] = lo;
+                h.bq[s] = hi;
+                h.bq_lo[s] = lo;
             } else {
                 uint4v w = *reinterpret_cast<const uint4v*>(static_cast<const uint16_t*>(p.q) +
                                                             off + 32 * s);
                 if (!q_valid) w = uint4v{0, 0, 0, 0};
-                bq[s] = as_half8(w);
+                h.bq[s] = as_half8(w);
             }
         }
     };
 
-    float m_run = kNegBig, l_run = 0.0f;
-    float4v acc[8];
-#pragma unroll
-    for (int t = 0; t < 8; t++) acc[t] = float4v{0, 0, 0, 0};
-
-    auto compute = [&](const TileRegs& r, const Cursor& c) {
+    auto compute = [&](const TileRegs& r, const Cursor& c, HeadState& h) {
         const uint32_t tok0 = c.t * kTile;
         float4v c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], bq[s], c0, 0, 0, 0);
-            c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], bq[s], c1, 0, 0, 0);
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], h.bq[s], c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], h.bq[s], c1, 0, 0, 0);
             if constexpr (kQF32) {
-                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], bq_lo[s], c0, 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], bq_lo[s], c1, 0, 0, 0);
+                c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], h.bq_lo[s], c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], h.bq_lo[s], c1, 0, 0, 0);
             }
         }
         float s[8];
@@ -244,16 +274,16 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
                            fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
         mloc = fmaxf(mloc, wave_shfl_xor(mloc, 16));
         mloc = fmaxf(mloc, wave_shfl_xor(mloc, 32));
-        const float m_new = fmaxf(m_run, mloc);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
+        const float m_new = fmaxf(h.m_run, mloc);
+        const float alpha = fast_exp2(h.m_run - m_new);
+        h.m_run = m_new;
         float psum = 0.0f, pj[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             pj[j] = fast_exp2(s[j] - m_new);
             psum += pj[j];
         }
-        l_run = l_run * alpha + psum;
+        h.l_run = h.l_run * alpha + psum;
         uint4v bpw;
         bpw.x = pack_f16x2(pj[0], pj[1]);
         bpw.y = pack_f16x2(pj[2], pj[3]);
@@ -268,21 +298,22 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
             aw.y = __builtin_amdgcn_perm(r.vr[3][t >> 1], r.vr[2][t >> 1], sel);
             aw.z = __builtin_amdgcn_perm(r.vr[5][t >> 1], r.vr[4][t >> 1], sel);
             aw.w = __builtin_amdgcn_perm(r.vr[7][t >> 1], r.vr[6][t >> 1], sel);
-            float4v cin = acc[t] * alpha;
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(aw), bp, cin, 0, 0, 0);
+            float4v cin = h.acc[t] * alpha;
+            h.acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(aw), bp, cin, 0, 0, 0);
         }
     };
 
-    // Writes the partial of the (sequence, head) the cursor is in and clears the state.
-    auto flush = [&](const Cursor& c) {
-        float l = l_run;
+    // Writes the partial of virtual head `vh` for the (sequence, list head) the cursor is
+    // in and clears the state.
+    auto flush = [&](const Cursor& c, uint32_t vh, HeadState& h) {
+        float l = h.l_run;
         l += wave_shfl_xor(l, 16);
         l += wave_shfl_xor(l, 32);
-        const uint32_t kvh = c.vh / p.q_groups, qg = c.vh % p.q_groups;
+        const uint32_t kvh = vh / p.q_groups, qg = vh % p.q_groups;
         const uint32_t q_in_group = qg * 16 + n;
         if (q_in_group < p.group) {
-            // slot = this worker's rank among the workers that touch (b, vh)
-            const uint32_t u_start = prefix_u(c.b) * vheads + c.vh * c.nt;
+            // slot = this worker's rank among the workers that touch (b, list head)
+            const uint32_t u_start = prefix_u(c.b) * lists + c.vh * c.nt;
             const uint32_t slot = worker - u_start / per;
             const size_t head = size_t(c.b) * p.num_heads + kvh * p.group + q_in_group;
             const size_t at = head * p.max_chunks + slot;
@@ -293,76 +324,115 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 2) decode_stream_kernel(De
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
                     const int e = 4 * i + k;  // d = 32g + e  <->  acc[e % 8][e / 8]
-                    w[k] = acc[e & 7][e >> 3];
+                    w[k] = h.acc[e & 7][e >> 3];
                 }
                 *reinterpret_cast<float4v*>(po + 4 * i) = w;
             }
             if (g == 0) {
-                p.part_ml[at * 2 + 0] = m_run;
+                p.part_ml[at * 2 + 0] = h.m_run;
                 p.part_ml[at * 2 + 1] = l;
             }
         }
-        m_run = kNegBig;
-        l_run = 0.0f;
-#pragma unroll
-        for (int t = 0; t < 8; t++) acc[t] = float4v{0, 0, 0, 0};
+        clear(h);
     };
 
-    // ---- three-stage pipeline over the wave's tiles
+    // ---- three-stage pipeline over the worker's tiles
     Cursor cc = first;  // tile being computed
     Cursor cl = first;  // tile whose K/V rows are requested next
     Cursor cr = first;  // tile whose block-table rows are requested next
     TileRegs ra, rb;
 
-    uint32_t rows_a = rows_of(cr);
-    advance(p, s_len, cr, 1 < n_units);
-    uint32_t rows_b = rows_of(cr);
-    advance(p, s_len, cr, 2 < n_units);
-    issue(ra, rows_a, cl);
-    advance(p, s_len, cl, 1 < n_units);
-    load_q(cc);
+    if constexpr (kPair) {
+        // Buffer A always holds the wave's first head of a tile, buffer B its second; both
+        // use the same rows, so there is one block-table lookup per tile.
+        HeadState ha, hb;
+        clear(ha);
+        clear(hb);
+        uint32_t rows_t = rows_of(cr);  // of the tile whose K/V is requested next
+        advance(p, s_len, lists, cr, 1 < n_units);
+        uint32_t rows_n = rows_of(cr);  // of the tile after it
+        advance(p, s_len, lists, cr, 2 < n_units);
+        issue(ra, rows_t, head_of(cl, 0));
+        load_q(cc.b, head_of(cc, 0), ha);
+        load_q(cc.b, head_of(cc, 1), hb);
 
-    for (uint32_t i = 0; i < n_units; i += 2) {
-        // tile i+1 (or tile i again at the very end) into buffer B
-        issue(rb, rows_b, cl);
-        advance(p, s_len, cl, i + 2 < n_units);
-        rows_a = rows_of(cr);
-        advance(p, s_len, cr, i + 3 < n_units);
+        for (uint32_t i = 0; i < n_units; i++) {
+            issue(rb, rows_t, head_of(cl, 1));
+            advance(p, s_len, lists, cl, i + 1 < n_units);
+            compute(ra, cc, ha);
 
-        compute(ra, cc);
-        {
+            rows_t = rows_n;
+            rows_n = rows_of(cr);
+            advance(p, s_len, lists, cr, i + 3 < n_units);
+            issue(ra, rows_t, head_of(cl, 0));  // tile i + 1 (tile i again at the very end)
+            compute(rb, cc, hb);
+
             const bool last = i + 1 >= n_units;
             const bool seg_end = last || cc.t + 1 == cc.nt;
             const Cursor done = cc;
-            advance(p, s_len, cc, !last);
+            advance(p, s_len, lists, cc, !last);
             if (seg_end) {
-                flush(done);
-                if (!last) load_q(cc);
+                flush(done, head_of(done, 0), ha);
+                flush(done, head_of(done, 1), hb);
+                if (!last) {
+                    load_q(cc.b, head_of(cc, 0), ha);
+                    load_q(cc.b, head_of(cc, 1), hb);
+                }
             }
-            if (last) break;
         }
+    } else {
+        HeadState h;
+        clear(h);
+        uint32_t rows_a = rows_of(cr);
+        advance(p, s_len, lists, cr, 1 < n_units);
+        uint32_t rows_b = rows_of(cr);
+        advance(p, s_len, lists, cr, 2 < n_units);
+        issue(ra, rows_a, cl.vh);
+        advance(p, s_len, lists, cl, 1 < n_units);
+        load_q(cc.b, cc.vh, h);
 
-        issue(ra, rows_a, cl);
-        advance(p, s_len, cl, i + 3 < n_units);
-        rows_b = rows_of(cr);
-        advance(p, s_len, cr, i + 4 < n_units);
+        for (uint32_t i = 0; i < n_units; i += 2) {
+            // tile i+1 (or tile i again at the very end) into buffer B
+            issue(rb, rows_b, cl.vh);
+            advance(p, s_len, lists, cl, i + 2 < n_units);
+            rows_a = rows_of(cr);
+            advance(p, s_len, lists, cr, i + 3 < n_units);
 
-        compute(rb, cc);
-        {
-            const bool last = i + 2 >= n_units;
-            const bool seg_end = last || cc.t + 1 == cc.nt;
-            const Cursor done = cc;
-            advance(p, s_len, cc, !last);
-            if (seg_end) {
-                flush(done);
-                if (!last) load_q(cc);
+            compute(ra, cc, h);
+            {
+                const bool last = i + 1 >= n_units;
+                const bool seg_end = last || cc.t + 1 == cc.nt;
+                const Cursor done = cc;
+                advance(p, s_len, lists, cc, !last);
+                if (seg_end) {
+                    flush(done, done.vh, h);
+                    if (!last) load_q(cc.b, cc.vh, h);
+                }
+                if (last) break;
+            }
+
+            issue(ra, rows_a, cl.vh);
+            advance(p, s_len, lists, cl, i + 3 < n_units);
+            rows_b = rows_of(cr);
+            advance(p, s_len, lists, cr, i + 4 < n_units);
+
+            compute(rb, cc, h);
+            {
+                const bool last = i + 2 >= n_units;
+                const bool seg_end = last || cc.t + 1 == cc.nt;
+                const Cursor done = cc;
+                advance(p, s_len, lists, cc, !last);
+                if (seg_end) {
+                    flush(done, done.vh, h);
+                    if (!last) load_q(cc.b, cc.vh, h);
+                }
             }
         }
     }
 }
 
 // Merges the partials of one (sequence, query head): the workers that touched
-// it are consecutive, first = u_start / per, last = (u_end - 1) / per.
+// its list head are consecutive, first = u_start / per, last = (u_end - 1) / per.
 __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodeParams p) {
     const uint32_t qh = blockIdx.x;
     const uint32_t b = blockIdx.y;
@@ -372,8 +442,9 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
     const uint32_t per = p.plan[0];
     const uint32_t vheads = p.num_kv_heads * p.q_groups;
     const uint32_t kvh = qh / p.group, qg = (qh % p.group) / 16;
-    const uint32_t vh = kvh * p.q_groups + qg;
-    const uint32_t u_start = prefix[b] * vheads + vh * nt;
+    const uint32_t heads_per_list = p.plan[2];  // 1 (flat list) or 8 (rows)
+    const uint32_t vh = (kvh * p.q_groups + qg) / heads_per_list;
+    const uint32_t u_start = prefix[b] * (vheads / heads_per_list) + vh * nt;
     const uint32_t n_parts = (u_start + nt - 1) / per - u_start / per + 1;
     const size_t head = size_t(b) * p.num_heads + qh;
     const float* ml = p.part_ml + head * p.max_chunks * 2;
@@ -398,11 +469,13 @@ bool decode_stream_supports(uint32_t batch) { return batch + 1 <= kStreamMaxPref
 
 int launch_decode_stream(DecodeParams p, bool q_f32, int rows) {
     if (!decode_stream_supports(p.batch)) return GRANITE_HIP_EINVAL;
-    // Workers: one wave per SIMD on every CU.
+    // One workgroup per CU, one wave per SIMD.  A worker is a workgroup when the heads come
+    // in groups of 8 (the rows shape), else a wave.
     const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
     const uint32_t wgs = cus;
-    const uint32_t workers = wgs * kWavesPerWG;
-    // Smallest range a wave may get: it bounds the partial slots per (sequence, head) to
+    const bool pair = (p.num_kv_heads * p.q_groups) % kPairHeads == 0;
+    const uint32_t workers = pair ? wgs : wgs * kWavesPerWG;
+    // Smallest range a worker may get: it bounds the partial slots per (sequence, head) to
     // about 32 however short the batch is, and is never above chunk_tokens.
     const uint32_t max_tiles = (p.max_tokens + kTile - 1) / kTile;
     const uint32_t min_per = min(max(p.chunk_tokens / kTile, 1u), max((max_tiles + 31) / 32, 1u));
@@ -427,9 +500,13 @@ int launch_decode_stream(DecodeParams p, bool q_f32, int rows) {
     {
         KernelTimerScope timer("decode_stream");
         dim3 grid(wgs), block(kWavesPerWG * kWave);
-#define GHIP_STREAM_CASE(QF32, ROWS)                               \
-    if (q_f32 == QF32 && rows == ROWS)                             \
-        decode_stream_kernel<QF32, ROWS><<<grid, block, lds_bytes, st>>>(p);
+#define GHIP_STREAM_CASE(QF32, ROWS)                                             \
+    if (q_f32 == QF32 && rows == ROWS) {                                         \
+        if (pair)                                                                \
+            decode_stream_kernel<QF32, ROWS, true><<<grid, block, lds_bytes, st>>>(p);  \
+        else                                                                     \
+            decode_stream_kernel<QF32, ROWS, false><<<grid, block, lds_bytes, st>>>(p); \
+    }
         GHIP_STREAM_CASE(true, kRowsContiguous)
         GHIP_STREAM_CASE(true, kRowsPagedPow2)
         GHIP_STREAM_CASE(true, kRowsPagedAny)
