@@ -79,6 +79,22 @@ def test_batched_paged_decode_small(gpu, oracle, q_dtype, bs):
     assert np.all(got[~live] == -7.0) and np.all(got_lse[~live] == -7.0)   # empty sequence untouched
 
 
+@pytest.mark.parametrize("hq,hkv", [(12, 3), (64, 16), (40, 2), (160, 8), (8, 8), (6, 1)])
+def test_batched_paged_decode_head_shapes(gpu, oracle, hq, hkv):
+    """Head counts on both sides of the kernel's two list shapes (heads in groups of 8 or
+    not), with more than 16 query heads per KV head among them."""
+    lens = np.array([40, 1300, 0, 31, 513, 2100, 64, 9], np.int32)
+    case = W.make_paged_decode(seed=hq, num_heads=hq, num_kv_heads=hkv, ctx_max=2112, seq_lens=lens)
+    say(f"batched paged decode heads hq={hq} hkv={hkv}")
+    want, want_lse = oracle.batched_paged_decode(case.q.astype(np.float32), case.k_pool, case.v_pool,
+                                                 case.block_tables, case.seq_lens, 16, case.scale)
+    got, got_lse = _run_batched(gpu, case, F16)
+    live = lens > 0
+    assert_close(got[live], want[live], "out")
+    assert_lse(got_lse[live], want_lse[live], "lse")
+    assert np.all(got[~live] == -7.0)
+
+
 @pytest.mark.parametrize("chunk", [32, 128, 512, 1024])
 def test_batched_paged_decode_chunk_sizes_agree(gpu, oracle, chunk):
     lens = np.array([900, 31, 1500, 1024], np.int32)
