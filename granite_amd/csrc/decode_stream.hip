@@ -195,7 +195,10 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const uint32_t row = lane_read(rows, tau(g, j));
-            r.vr[j] = *reinterpret_cast<const uint4v*>(vbase + size_t(row) * p.tok_stride);
+            // every byte of V is used once: a streaming load measured 9 % faster (for K,
+            // whose lines are covered by four instructions, it made no difference)
+            r.vr[j] = __builtin_nontemporal_load(
+                reinterpret_cast<const uint4v*>(vbase + size_t(row) * p.tok_stride));
         }
     };
 
