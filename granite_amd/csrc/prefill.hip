@@ -191,19 +191,34 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     const uint32_t gidx = job / members, member = job - gidx * members;
     const uint32_t split = gidx % p.n_splits;
     const uint32_t head = (gidx / p.n_splits) * p.group + member / p.q_tiles;
-    // heavy (late) query tiles first so the causal tail is short
-    const uint32_t q_tile = p.q_tiles - 1 - member % p.q_tiles;
     const uint32_t kvh = head / p.group;
-    const uint32_t q0_wg = q_tile * kBM;
-    const uint32_t q0 = q0_wg + 32 * wave;
+    // ---- the query rows.  A workgroup holds two runs of 128 rows (half tiles), one per four
+    // waves, so one per SIMD pair of waves.  Normally they are the two halves of query tile
+    // `slot` from the end.  Under a causal mask the work of a half tile grows with its
+    // position (4 .. 32 key tiles across 2048 tokens), so the k-th workgroup of a head takes
+    // the k-th half tile from the end and the k-th from the start instead: every workgroup
+    // then has the same number of (wave, key tile) steps, and while only the late half tile
+    // still has keys to visit its waves have their SIMDs to themselves.
+    constexpr uint32_t kHalf = kBM / 2;
+    const uint32_t slot = member % p.q_tiles;
+    const uint32_t halves = (p.seq_q + kHalf - 1) / kHalf;
+    const bool paired = p.mask_mode == GRANITE_HIP_MASK_CAUSAL;
+    const uint32_t late_half = paired ? halves - 1 - slot : 2 * (p.q_tiles - 1 - slot) + 1;
+    const uint32_t early_half = paired ? slot : late_half - 1;
+    // (an odd count leaves the middle half tile alone in its workgroup)
+    const bool second_run = wave >= kThreads / 128;
+    const bool run_live = !second_run || early_half < late_half;
+    const uint32_t my_half = paired ? (second_run ? early_half : late_half)
+                                    : (second_run ? late_half : early_half);
+    const uint32_t q0 = run_live ? my_half * kHalf + 32 * (wave & 3) : p.seq_q;
     const uint32_t q_row = q0 + n;
     const bool wave_active = q0 < p.seq_q;
     const uint32_t q_ld = min(q_row, p.seq_q - 1);
 
-    // ---- keys this workgroup has to visit
+    // ---- keys this workgroup has to visit: those of its later half tile
     uint32_t len_a = p.cache_len;
     if (p.mask_mode == GRANITE_HIP_MASK_CAUSAL) {
-        const uint32_t q_last = min(q0_wg + kBM, p.seq_q) - 1;
+        const uint32_t q_last = min((late_half + 1) * kHalf, p.seq_q) - 1;
         len_a = min(len_a, p.start_pos + q_last + 1);
     }
     const uint32_t len_b = p.extra_len;
