@@ -47,9 +47,9 @@ CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
 # `--workload copy_calibration` (1.998 KiB per FETCH_SIZE unit, 1.000 KiB per
 # WRITE_SIZE unit); the summaries are under profiles/.
 MEASURED_TRAFFIC = {
-    "paged_decode": 1134673288,    # decode_stream_kernel; algorithmic 1132236296
-    "prefill": 42546817,           # attention_tiles_kernel; algorithmic 41943040
-    "chunked_prefill": 179564192,  # attention_tiles_kernel; algorithmic 153092096
+    "paged_decode": 1146033048,    # decode_stream_kernel; algorithmic 1132236296
+    "prefill": 42557968,           # attention_tiles_kernel; algorithmic 41943040
+    "chunked_prefill": 179300866,  # attention_tiles_kernel; algorithmic 153092096
 }
 
 
