@@ -386,12 +386,93 @@ def bench_copy_calibration(gpu, steps, warmup, cpu):
             "parity": {"bit_exact": bool(np.array_equal(got, np.transpose(pool, (1, 0, 2))))}}
 
 
+def bench_rope_append(gpu, steps, warmup, cpu):
+    """The step in front of the attention path: rotate Q and K (the reference's cos/sin tables
+    as input) and append the rotated K and V to the paged cache in the same pass.  Shape: a
+    prefill of 8192 tokens, 64 query heads, 8 KV heads, block 32 (the chunk of the chunked
+    prefill config, 512 tokens at position 32768, is timed beside it: it is launch bound)."""
+    from granite_amd import DeviceBuffer, ROUND_NEAREST
+    dev = DeviceBuffer.from_numpy
+    hq, hkv, d, bs = 64, 8, 128, 32
+    import oracle_bind
+    oracle = oracle_bind.load() if cpu else None
+
+    def make(seq, start, seed):
+        rng = np.random.default_rng(seed)
+        q = rng.standard_normal((seq, hq, d), dtype=np.float32)
+        k = rng.standard_normal((seq, hkv, d), dtype=np.float32)
+        v = rng.standard_normal((seq, hkv, d), dtype=np.float32)
+        positions = start + seq
+        i = np.arange(d // 2, dtype=np.float32)
+        freq = (1.0 / np.float32(10000.0) ** (2 * i / np.float32(d))).astype(np.float32)
+        ang = (np.arange(positions, dtype=np.float32)[:, None] * freq[None, :]).astype(np.float32)
+        cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+        if oracle is not None:  # the reference's own table (libm in float)
+            cos, sin = oracle.rope_table(positions, d, 10000.0)
+        nblk = (positions + bs - 1) // bs
+        table = rng.permutation(nblk).astype(np.int32)
+        bufs = dict(q=dev(q), k=dev(k), v=dev(v), cos=dev(cos), sin=dev(sin), t=dev(table),
+                    pk=dev(np.zeros((nblk * bs, hkv, d), np.uint16)),
+                    pv=dev(np.zeros((nblk * bs, hkv, d), np.uint16)))
+        host = dict(q=q, k=k, v=v, cos=cos, sin=sin, table=table, nblk=nblk)
+
+        def step():
+            gpu.rope_append(seq_len=seq, head_dim=d, start_pos=start, q=bufs["q"], num_heads_q=hq,
+                            k=bufs["k"], num_heads_k=hkv, v=bufs["v"], cache_k=bufs["pk"], cache_v=bufs["pv"],
+                            block_table=bufs["t"], block_size=bs, cos_table=bufs["cos"], sin_table=bufs["sin"],
+                            table_positions=positions, write_k_back=False, rounding=ROUND_NEAREST)
+        # Q read and written, K and V read, two half cache rows written, the cos/sin rows read
+        nbytes = seq * (2 * hq * d * 4 + 2 * hkv * d * 4 + 2 * hkv * d * 2 + 2 * (d // 2) * 4)
+        return step, bufs, host, nbytes
+
+    step, bufs, host, nbytes = make(8192, 0, 21)
+    ms, wall_ms, kern = Timer(gpu).run(step, warmup, steps)
+    c_step, _, _, c_bytes = make(512, 32768, 22)
+    c_ms, _, c_kern = Timer(gpu).run(c_step, warmup, steps)
+    res = {
+        "workload": "rope_append_s8192_hq64_hkv8_d128_bs32", "metric": "rope_append_GBps", "unit": "GB/s",
+        "value": round(nbytes / (ms * 1e-3) / 1e9, 1), "ms_per_step": round(ms, 4),
+        "wall_ms_per_step": round(wall_ms, 4), "algorithmic_bytes": nbytes, "dtype": "f32 rotation, f16 cache",
+        "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
+        "chunk_512_at_32768": {"ms_per_step": round(c_ms, 4), "algorithmic_bytes": c_bytes,
+                               "GBps": round(c_bytes / (c_ms * 1e-3) / 1e9, 1)},
+        "note": "Q is rotated in place once per timed step (the values keep turning; the traffic is the same)",
+    }
+    res["roofline"] = roofline("hbm", nbytes, kern["rope_append"][0], None)
+    res["roofline"]["kernel"] = "rope_append_kernel"
+    if cpu:
+        # parity on a fresh copy: one application against the oracle, bit for bit
+        seq = 8192
+        fresh_q, fresh_k = dev(host["q"]), dev(host["k"])
+        gpu.rope_append(seq_len=seq, head_dim=d, start_pos=0, q=fresh_q, num_heads_q=hq, k=fresh_k,
+                        num_heads_k=hkv, v=bufs["v"], cache_k=bufs["pk"], cache_v=bufs["pv"],
+                        block_table=bufs["t"], block_size=bs, cos_table=bufs["cos"], sin_table=bufs["sin"],
+                        table_positions=seq, write_k_back=True, rounding=ROUND_NEAREST)
+        gpu.sync()
+        passes, t0 = 0, time.perf_counter()
+        while passes == 0 or time.perf_counter() - t0 < CPU_SAMPLE_SECONDS:
+            want_q = oracle.rope_apply(host["q"], 0, host["cos"], host["sin"])
+            want_k = oracle.rope_apply(host["k"], 0, host["cos"], host["sin"])
+            passes += 1
+        cpu_s = (time.perf_counter() - t0) / passes
+        rows = host["table"][np.arange(seq) // bs] * bs + np.arange(seq) % bs
+        pool_k = bufs["pk"].read(np.uint16, (host["nblk"] * bs, hkv, d))
+        res["cpu_baseline"] = {"value": round(seq * (2 * hq * d * 4 + 2 * hkv * d * 4) / cpu_s / 1e9, 3), "unit": "GB/s",
+                               "cores": 1, "kind": "port", "seconds": round(cpu_s * passes, 2),
+                               "sample": f"the rotation of Q and K of the whole workload (no append), mean of {passes} passes"}
+        res["parity"] = {"q_bit_exact": bool(np.array_equal(fresh_q.read(np.float32, host["q"].shape), want_q)),
+                         "k_bit_exact": bool(np.array_equal(fresh_k.read(np.float32, host["k"].shape), want_k)),
+                         "k_cache_bit_exact": bool(np.array_equal(pool_k[rows], want_k.astype(np.float16).view(np.uint16)))}
+    return res
+
+
 WORKLOADS = {
     "paged_decode": bench_paged_decode,
     "prefill": bench_prefill,
     "chunked_prefill": bench_chunked_prefill,
     "tree": bench_tree,
     "decode_contiguous": bench_decode_contiguous,
+    "rope_append": bench_rope_append,
 }
 EXTRA_WORKLOADS = {"copy_calibration": bench_copy_calibration}
 

@@ -94,6 +94,31 @@ class AttentionArgs(C.Structure):
     ]
 
 
+class RopeArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p),
+        ("q_f16", C.c_void_p),
+        ("k", C.c_void_p),
+        ("v", C.c_void_p),
+        ("cache_k", C.c_void_p),
+        ("cache_v", C.c_void_p),
+        ("block_table", C.c_void_p),
+        ("cos_table", C.c_void_p),
+        ("sin_table", C.c_void_p),
+        ("table_positions", C.c_uint32),
+        ("num_heads_q", C.c_uint32),
+        ("num_heads_k", C.c_uint32),
+        ("seq_len", C.c_uint32),
+        ("head_dim", C.c_uint32),
+        ("start_pos", C.c_uint32),
+        ("max_seq_len", C.c_uint32),
+        ("block_size", C.c_uint32),
+        ("freq_base", C.c_float),
+        ("write_k_back", C.c_int),
+        ("rounding", C.c_int),
+    ]
+
+
 _u32, _i64, _vp, _int, _f32 = C.c_uint32, C.c_int64, C.c_void_p, C.c_int, C.c_float
 
 # name -> (restype, argtypes); every symbol granite_hip.h declares
@@ -141,6 +166,8 @@ SIGNATURES = {
     "granite_hip_decode_attention": (_int, [C.POINTER(DecodeArgs)]),
     "granite_hip_attention": (_int, [C.POINTER(AttentionArgs)]),
     "granite_hip_build_tree_mask": (_int, [_vp, _vp, _u32]),
+    "granite_hip_rope_multihead": (_int, [_vp, _vp, _u32, _u32, _u32, _u32, _u32, _f32]),
+    "granite_hip_rope_append": (_int, [C.POINTER(RopeArgs)]),
     "granite_hip_workspace_bytes": (C.c_size_t, []),
 }
 

@@ -297,6 +297,32 @@ int granite_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
     return GRANITE_HIP_OK;
 }
 
+// ---- RoPE (+ append) -----------------------------------------------------
+
+int granite_hip_rope_append(const granite_hip_rope_args* args) {
+    GHIP_REQUIRE_INIT();
+    if (!args) return GRANITE_HIP_ENULL;
+    return ghip::launch_rope_append(*args);
+}
+
+int granite_hip_rope_multihead(void* q, void* k, uint32_t num_heads_q, uint32_t num_heads_k,
+                               uint32_t seq_len, uint32_t head_dim, uint32_t start_pos,
+                               float freq_base) {
+    GHIP_REQUIRE_INIT();
+    granite_hip_rope_args a{};
+    a.q = q;
+    a.k = k;
+    a.num_heads_q = num_heads_q;
+    a.num_heads_k = num_heads_k;
+    a.seq_len = seq_len;
+    a.head_dim = head_dim;
+    a.start_pos = start_pos;
+    a.freq_base = freq_base;
+    a.write_k_back = 1;
+    a.rounding = GRANITE_HIP_ROUND_TRUNCATE;
+    return ghip::launch_rope_append(a);
+}
+
 size_t granite_hip_workspace_bytes(void) { return ctx().workspace_bytes; }
 
 int granite_hip_enable_kernel_timing(int enable) {

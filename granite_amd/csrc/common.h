@@ -76,6 +76,7 @@ int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const 
 int launch_decode(const granite_hip_decode_args& a);
 int launch_attention(const granite_hip_attention_args& a);
 int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes);
+int launch_rope_append(const granite_hip_rope_args& a);
 
 // ---- device helpers ------------------------------------------------------
 #if defined(__HIPCC__)
@@ -83,6 +84,7 @@ int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));

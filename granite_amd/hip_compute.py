@@ -14,7 +14,7 @@ import numpy as np
 
 from . import _capi
 from ._capi import (F16, F32, MASK_CAUSAL, MASK_NONE, MASK_TREE, MEM_DEVICE, ROUND_NEAREST,
-                    ROUND_TRUNCATE, AttentionArgs, DecodeArgs, check)
+                    ROUND_TRUNCATE, AttentionArgs, RopeArgs, DecodeArgs, check)
 
 
 class DeviceBuffer:
@@ -231,6 +231,29 @@ class HipCompute:
                           start_pos=start_pos, seq_q=seq_q, num_heads=num_heads,
                           num_kv_heads=num_kv_heads, head_dim=head_dim, scale=scale)
         check(self.lib.granite_hip_attention(C.byref(a)), "attention")
+
+    def rope_multihead(self, q, k, num_heads_q, num_heads_k, seq_len, head_dim, start_pos,
+                       freq_base=10000.0) -> None:
+        """MetalCompute::rope_multihead (include/granite/metal_compute.h:728-739): q
+        [seq, Hq, D] and k [seq, Hkv, D] float, rotated in place."""
+        check(self.lib.granite_hip_rope_multihead(_p(q), _p(k), num_heads_q, num_heads_k, seq_len,
+                                                  head_dim, start_pos, freq_base), "rope_multihead")
+
+    def rope_append(self, *, seq_len, head_dim, start_pos, q=None, num_heads_q=0, q_f16=None, k=None,
+                    num_heads_k=0, v=None, cache_k=None, cache_v=None, block_table=None, block_size=0,
+                    max_seq_len=0, cos_table=None, sin_table=None, table_positions=0,
+                    freq_base=10000.0, write_k_back=True, rounding=ROUND_TRUNCATE) -> None:
+        """Rotation of Q and K and, in the same pass, the append of the rotated K and of V to
+        the (contiguous or paged) half cache; with RoPECache's tables the rotation is
+        bit-identical to RoPECache::apply (src/llm/rope.cpp:24-92)."""
+        a = RopeArgs(q=_p(q), q_f16=_p(q_f16), k=_p(k), v=_p(v), cache_k=_p(cache_k),
+                     cache_v=_p(cache_v), block_table=_p(block_table), cos_table=_p(cos_table),
+                     sin_table=_p(sin_table), table_positions=table_positions,
+                     num_heads_q=num_heads_q, num_heads_k=num_heads_k, seq_len=seq_len,
+                     head_dim=head_dim, start_pos=start_pos, max_seq_len=max_seq_len,
+                     block_size=block_size, freq_base=freq_base, write_k_back=int(write_k_back),
+                     rounding=rounding)
+        check(self.lib.granite_hip_rope_append(C.byref(a)), "rope_append")
 
     def build_tree_mask(self, parent_indices, mask_words, num_nodes) -> None:
         check(self.lib.granite_hip_build_tree_mask(_p(parent_indices), _p(mask_words), num_nodes),

@@ -13,6 +13,7 @@
 
 struct granite_hip_attention_args;
 struct granite_hip_decode_args;
+struct granite_hip_rope_args;
 
 namespace granite {
 
@@ -76,6 +77,14 @@ class HipCompute {
                                  const HipBuffer* V_cache, const HipBuffer* block_table,
                                  uint32_t num_kv_heads, uint32_t head_dim, uint32_t len,
                                  uint32_t block_size, uint32_t max_seq_len);
+
+    // MetalCompute::rope_multihead (include/granite/metal_compute.h:728-739): q [seq, Hq, D]
+    // and k [seq, Hkv, D] float, rotated in place, cos/sin evaluated on the device.
+    Result<void> rope_multihead(HipBuffer* q, HipBuffer* k, uint32_t num_heads_q,
+                                uint32_t num_heads_k, uint32_t seq_len, uint32_t head_dim,
+                                uint32_t start_pos, float freq_base = 10000.0f);
+    // The rotation (from cos/sin tables or evaluated) fused with the K/V append.
+    Result<void> rope_append(const granite_hip_rope_args& args);
 
     // General entry points (strided Q/out, fp16 or fp32, paged or contiguous
     // keys, causal / tree masks, optional log-sum-exp).

@@ -150,6 +150,17 @@ Result<void> HipCompute::paged_kv_gather(HipBuffer* dst_k, HipBuffer* dst_v,
                                                 max_seq_len));
 }
 
+Result<void> HipCompute::rope_multihead(HipBuffer* q, HipBuffer* k, uint32_t num_heads_q,
+                                        uint32_t num_heads_k, uint32_t seq_len, uint32_t head_dim,
+                                        uint32_t start_pos, float freq_base) {
+    return HIP_CALL(granite_hip_rope_multihead(q, k, num_heads_q, num_heads_k, seq_len, head_dim,
+                                               start_pos, freq_base));
+}
+
+Result<void> HipCompute::rope_append(const granite_hip_rope_args& args) {
+    return HIP_CALL(granite_hip_rope_append(&args));
+}
+
 Result<void> HipCompute::attention(const granite_hip_attention_args& args) {
     return HIP_CALL(granite_hip_attention(&args));
 }

@@ -3,6 +3,7 @@
 // pools) and SpeculationTree.  The KVCache cases repeat the reference's own
 // (tests/test_llm.cpp:113-160) on a host-memory test double.
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 
 #include "check.h"
@@ -10,6 +11,7 @@
 #include "granite/hip_compute.h"
 #include "granite/kv_cache.h"
 #include "granite/operators.h"
+#include "granite/rope.h"
 #include "granite_hip.h"
 #include "host_memory_backend.h"
 
@@ -496,6 +498,47 @@ TEST_CASE(factory_knows_only_hip) {
     CHECK(hip_device_pointer(nullptr, BufferHandle{1}) == nullptr);
     HostMemoryBackend be;
     CHECK(hip_device_pointer(&be, BufferHandle{1}) == nullptr);
+}
+
+extern "C" void go_rope_table(float* cos_out, float* sin_out, int max_seq_len, int head_dim, float theta);
+
+TEST_CASE(rope_cache_tables_and_checks) {
+    // tests/test_llm.cpp:14-63 of the reference: sizes, position 0, position 1
+    RoPECache cache;
+    CHECK(!cache.is_initialized());
+    cache.initialize(2048, 64, 10000.0f);
+    CHECK(cache.is_initialized());
+    CHECK(cache.cos_cache().size() == size_t(2048) * 32);
+    CHECK(cache.sin_cache().size() == size_t(2048) * 32);
+    RoPECache small;
+    small.initialize(1024, 8, 10000.0f);
+    for (int i = 0; i < 4; ++i) {
+        CHECK(std::fabs(small.cos_cache()[i] - 1.0f) <= 1e-5f);
+        CHECK(std::fabs(small.sin_cache()[i]) <= 1e-5f);
+        const float angle = 1.0f / std::pow(10000.0f, static_cast<float>(2 * i) / 8);
+        CHECK(std::fabs(small.cos_cache()[4 + i] - std::cos(angle)) <= 1e-5f);
+        CHECK(std::fabs(small.sin_cache()[4 + i] - std::sin(angle)) <= 1e-5f);
+    }
+    // same bits as the oracle's table
+    std::vector<float> c(size_t(1024) * 4), s(c.size());
+    go_rope_table(c.data(), s.data(), 1024, 8, 10000.0f);
+    CHECK(small.cos_cache() == c);
+    CHECK(small.sin_cache() == s);
+
+    // argument checks come before anything touches a device
+    HostMemoryBackend be;
+    REQUIRE(be.initialize().ok());
+    Tensor q = Tensor::allocate({1, 4, 2, 8}, DataType::FP32, &be).take();
+    Tensor k = Tensor::allocate({1, 4, 1, 8}, DataType::FP32, &be).take();
+    RoPECache none;
+    CHECK_CODE(none.apply(q, k, 0, &be), ErrorCode::InvalidState);
+    CHECK_CODE(small.apply(q, k, 1021, &be), ErrorCode::InvalidArgument);  // 1021 + 4 > 1024
+    Tensor wrong_dim = Tensor::allocate({1, 4, 2, 16}, DataType::FP32, &be).take();
+    CHECK_CODE(small.apply(wrong_dim, k, 0, &be), ErrorCode::ShapeMismatch);
+    Tensor half_q = Tensor::allocate({1, 4, 2, 8}, DataType::FP16, &be).take();
+    CHECK_CODE(small.apply(half_q, k, 0, &be), ErrorCode::DTypeMismatch);
+    // a backend that is not the GPU is refused, never computed on the host
+    CHECK_CODE(small.apply(q, k, 0, &be), ErrorCode::BackendNotSupported);
 }
 
 int main(int argc, char** argv) { return hosttest::run_all(argc, argv); }

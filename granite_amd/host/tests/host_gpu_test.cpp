@@ -11,6 +11,7 @@
 #include "granite/hip_compute.h"
 #include "granite/kv_cache.h"
 #include "granite/operators.h"
+#include "granite/rope.h"
 #include "granite_hip.h"
 
 extern "C" {
@@ -30,6 +31,9 @@ void go_batched_paged_decode(const float* q, const uint16_t* pool_k, const uint1
                              const int32_t* tables, const int32_t* seq_lens, float* out, float* lse,
                              int batch, int num_heads, int num_kv_heads, int head_dim,
                              int block_size, int max_blocks, float scale);
+void go_rope_table(float* cos_out, float* sin_out, int max_seq_len, int head_dim, float theta);
+int go_rope_apply(float* x, int seq_len, int num_heads, int head_dim, int start_pos, const float* cos_t,
+                  const float* sin_t, int max_seq_len);
 int go_attention_tree(const float* q, const uint16_t* cache_k, const uint16_t* cache_v,
                       const int32_t* table, int block_size, int max_seq, const float* k_tree,
                       const float* v_tree, const int32_t* parent, float* context, float* lse,
@@ -461,6 +465,84 @@ TEST_CASE(speculation_tree_attention) {
             std::memcpy(&want[(size_t(h) * N + n) * D], &want_tok[(size_t(n) * H + h) * D], D * 4);
     CHECK(close_enough(got, want, "tree attention over SpeculationTree parents"));
     for (HipBuffer* p : {d_q, d_ck, d_cv, d_tk, d_tv, d_p, d_o}) hc->release_buffer(p);
+}
+
+// float -> half, round to nearest even (what the GPU path's conversion does)
+uint16_t half_nearest(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint16_t sign = static_cast<uint16_t>((x >> 16) & 0x8000u);
+    x &= 0x7FFFFFFFu;
+    if (x > 0x7F800000u) return sign | 0x7E00u;
+    if (x >= 0x477FF000u) return sign | 0x7C00u;  // 65520 and above round to infinity
+    if (x < 0x38800000u) {                         // below the smallest normal half
+        if (x < 0x33000000u) return sign;          // at most half of the smallest subnormal
+        const int shift = 126 - static_cast<int>(x >> 23);
+        const uint32_t m = (x & 0x7FFFFFu) | 0x800000u;
+        uint32_t h = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1), half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (h & 1u))) ++h;
+        return sign | static_cast<uint16_t>(h);
+    }
+    uint32_t h = (x - 0x38000000u) >> 13;
+    const uint32_t rem = x & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+    return sign | static_cast<uint16_t>(h);
+}
+
+TEST_CASE(rope_cache_apply_and_append) {
+    REQUIRE(backend() != nullptr);
+    const int max_pos = 300, hq = 6, hkv = 2, seq = 21, start = 250;
+    RoPECache rope;
+    Tensor dummy = Tensor::allocate({1, 1, 1, D}, DataType::FP32, backend()).take();
+    CHECK_CODE(rope.apply(dummy, dummy, 0, backend()), ErrorCode::InvalidState);  // rope.cpp:25-27
+    rope.initialize(max_pos, D, 10000.0f);
+    REQUIRE(rope.is_initialized());
+    // the host tables are the reference's (and the oracle's) to the bit
+    std::vector<float> cos_t(size_t(max_pos) * D / 2), sin_t(cos_t.size());
+    go_rope_table(cos_t.data(), sin_t.data(), max_pos, D, 10000.0f);
+    CHECK(rope.cos_cache() == cos_t);
+    CHECK(rope.sin_cache() == sin_t);
+
+    auto q = randn(size_t(seq) * hq * D, 901), k = randn(size_t(seq) * hkv * D, 902),
+         v = randn(size_t(seq) * hkv * D, 903);
+    Tensor Q = upload({1, seq, hq, D}, DataType::FP32, q);
+    Tensor K = upload({1, seq, hkv, D}, DataType::FP32, k);
+    Tensor V = upload({1, seq, hkv, D}, DataType::FP32, v);
+    CHECK_OK(rope.apply(Q, K, start, backend()));
+    auto want_q = q, want_k = k;
+    CHECK(go_rope_apply(want_q.data(), seq, hq, D, start, cos_t.data(), sin_t.data(), max_pos) == 0);
+    CHECK(go_rope_apply(want_k.data(), seq, hkv, D, start, cos_t.data(), sin_t.data(), max_pos) == 0);
+    CHECK(download<float>(Q) == want_q);  // bit exact
+    CHECK(download<float>(K) == want_k);
+    // the range check of rope.cpp:34-38
+    CHECK_CODE(rope.apply(Q, K, max_pos - seq + 1, backend()), ErrorCode::InvalidArgument);
+
+    // rotate and append in one pass: cache rows are the rounded rotated K and V
+    const int max_len = 280;
+    Tensor K2 = upload({1, seq, hkv, D}, DataType::FP32, k);
+    Tensor Q2 = upload({1, seq, hq, D}, DataType::FP32, q);
+    std::vector<uint16_t> sentinel(size_t(hkv) * max_len * D, 0x1234);
+    Tensor CK = upload({hkv, max_len, D}, DataType::FP16, sentinel);
+    Tensor CV = upload({hkv, max_len, D}, DataType::FP16, sentinel);
+    CHECK_OK(rope.apply_and_append(Q2, K2, V, CK, CV, start, backend()));
+    CHECK(download<float>(Q2) == want_q);
+    auto got_k = download<uint16_t>(CK), got_v = download<uint16_t>(CV);
+    size_t wrong = 0;
+    for (int h = 0; h < hkv; ++h)
+        for (int pos = 0; pos < max_len; ++pos)
+            for (int d = 0; d < D; ++d) {
+                const size_t at = (size_t(h) * max_len + pos) * D + d;
+                uint16_t wk = 0x1234, wv = 0x1234;
+                if (pos >= start && pos < start + seq) {
+                    const size_t src = (size_t(pos - start) * hkv + h) * D + d;
+                    wk = half_nearest(want_k[src]);
+                    wv = half_nearest(v[src]);
+                }
+                wrong += (got_k[at] != wk) + (got_v[at] != wv);
+            }
+    CHECK(wrong == 0);
+    CHECK_CODE(rope.apply_and_append(Q2, K2, V, CK, CV, 270, backend()), ErrorCode::InvalidArgument);
 }
 
 int main(int argc, char** argv) {

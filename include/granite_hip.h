@@ -115,7 +115,7 @@ int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
  * reset_kernel_timing, get_kernel_timing_stats; include/granite/metal_compute.h:51-59).
  * While enabled every launch is bracketed by two events on the launch stream.
  * Names: "kv_append", "kv_gather", "decode_stream" or "decode_splitk",
- * "decode_merge", "attention_tiles", "attention_merge", "tree_mask".  granite_hip_kernel_timing_names() writes the
+ * "decode_merge", "attention_tiles", "attention_merge", "tree_mask", "rope_append".  granite_hip_kernel_timing_names() writes the
  * names seen so far, comma separated. */
 int granite_hip_enable_kernel_timing(int enable);
 int granite_hip_reset_kernel_timing(void);
@@ -296,6 +296,57 @@ int granite_hip_attention(const granite_hip_attention_args *args);
  * cannot hang the device. */
 int granite_hip_build_tree_mask(const int32_t *parent_indices, uint32_t *mask_words,
                                 uint32_t num_nodes);
+
+/* ---- rotary position embedding, fused with the K/V append ---------------- */
+
+/* MetalCompute::rope_multihead (include/granite/metal_compute.h:728-739;
+ * kernel src/backend/metal/kernels/metal_shaders_util.h:596-635): q
+ * [seq_len, num_heads_q, D] float and k [seq_len, num_heads_k, D] float are
+ * rotated in place, pairs (2i, 2i+1) by (start_pos + s) * freq_base^(-2i/D),
+ * cos/sin evaluated on the device in float as the reference kernel does. */
+int granite_hip_rope_multihead(void *q, void *k, uint32_t num_heads_q, uint32_t num_heads_k,
+                               uint32_t seq_len, uint32_t head_dim, uint32_t start_pos,
+                               float freq_base);
+
+/* General form: the rotation and, in the same pass, the append that follows it
+ * on the path (MetalCompute::kv_cache_append / paged_kv_cache_append above;
+ * call order src/llm/transformer.mm:3363 ff.).
+ *   q, k          as above; either may be NULL.  k is rewritten in float only
+ *                 when write_k_back is set (the reference always does).
+ *   q_f16         optional half copy of the rotated q, same layout, round to
+ *                 nearest (the dtype the prefill kernel reads directly)
+ *   v             [seq_len, num_heads_k, D] float, NULL without cache_v
+ *   cache_k/v     NULL: no append.  block_table NULL: contiguous cache
+ *                 [num_heads_k, max_seq_len, D] half, rows start_pos ..;
+ *                 else the paged pools [rows, num_heads_k, D] half
+ *   cos_table,    RoPECache's tables (src/llm/rope.cpp:5-22), float
+ *   sin_table     [table_positions, D/2] on the device: the rotation then uses
+ *                 exactly these values and separately rounded products, and is
+ *                 bit-identical to RoPECache::apply (rope.cpp:24-92); start_pos
+ *                 + seq_len > table_positions -> GRANITE_HIP_EOVERFLOW, its
+ *                 range check (rope.cpp:34-38).  Both NULL: evaluated from
+ *                 freq_base on the device.
+ *   rounding      float -> half conversion of the cache rows */
+typedef struct granite_hip_rope_args {
+    void *q;
+    void *q_f16;
+    void *k;
+    const void *v;
+    void *cache_k;
+    void *cache_v;
+    const int32_t *block_table;
+    const float *cos_table;
+    const float *sin_table;
+    uint32_t table_positions;
+    uint32_t num_heads_q, num_heads_k, seq_len, head_dim, start_pos;
+    uint32_t max_seq_len; /* contiguous cache */
+    uint32_t block_size;  /* paged */
+    float freq_base;
+    int write_k_back;
+    int rounding;
+} granite_hip_rope_args;
+
+int granite_hip_rope_append(const granite_hip_rope_args *args);
 
 /* Bytes of device scratch the library keeps for split-K partial results. */
 size_t granite_hip_workspace_bytes(void);

@@ -24,6 +24,8 @@
  *   go_attention_tree          src/llm/transformer.mm:1978-1983, 2012-2042, 2044-2126
  *   go_block_manager_*         src/llm/paged_kv_cache.cpp:17-98
  *   go_paged_cache_*           src/llm/paged_kv_cache.cpp:104-187
+ *   go_rope_table              src/llm/rope.cpp:5-22
+ *   go_rope_apply              src/llm/rope.cpp:24-92
  *
  * Pinning (what fixes each function besides re-reading it):
  *   conversions     all 65536 halves against the compiler's _Float16, the
@@ -38,6 +40,11 @@
  *                   lse = max_k s_k + ln sum_k exp(s_k - max), pinned by the
  *                   float64 implementation.
  *   block manager   closed forms (LIFO hand-out order N-1, N-2, ...).
+ *   rope            the reference's table tests (tests/test_llm.cpp:14-63: size,
+ *                   position 0 is (1, 0), position 1 against libm), a float64
+ *                   evaluation of the same fp32 angle, and what a rotation fixes:
+ *                   pair norms kept, position 0 is the identity, two rotations
+ *                   compose, a unit vector maps to (cos, sin).
  */
 #define _GNU_SOURCE
 #include <math.h>
@@ -701,4 +708,49 @@ int go_paged_cache_physical_block(const struct go_paged_cache *c, int pos)
 int go_paged_cache_block_offset(const struct go_paged_cache *c, int pos)
 {
     return pos % c->mgr->block_size;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Rotary position embedding                                                 */
+/* ------------------------------------------------------------------------- */
+
+/* RoPECache::initialize, src/llm/rope.cpp:5-22: cos/sin [max_seq_len, head_dim/2],
+ * freq = 1 / pow(theta, 2i / head_dim) and angle = pos * freq, all in float (the
+ * reference calls std::pow / std::cos / std::sin on float arguments). */
+void go_rope_table(float *cos_out, float *sin_out, int max_seq_len, int head_dim, float theta)
+{
+    int half_dim = head_dim / 2;
+    for (int pos = 0; pos < max_seq_len; pos++) {
+        for (int i = 0; i < half_dim; i++) {
+            float freq = 1.0f / powf(theta, (float)(2 * i) / head_dim);
+            float angle = (float)pos * freq;
+            cos_out[(size_t)pos * half_dim + i] = cosf(angle);
+            sin_out[(size_t)pos * half_dim + i] = sinf(angle);
+        }
+    }
+}
+
+/* RoPECache::apply, src/llm/rope.cpp:24-92, on one tensor [seq_len, num_heads, head_dim]
+ * (the reference runs the same loop over Q and then over K).  Returns -1 for the range
+ * error of rope.cpp:34-38. */
+int go_rope_apply(float *x, int seq_len, int num_heads, int head_dim, int start_pos,
+                  const float *cos_t, const float *sin_t, int max_seq_len)
+{
+    if (start_pos + seq_len > max_seq_len) return -1;
+    int half_dim = head_dim / 2;
+    for (int s = 0; s < seq_len; s++) {
+        int pos = start_pos + s;
+        for (int h = 0; h < num_heads; h++) {
+            float *p = x + ((size_t)s * num_heads + h) * head_dim;
+            for (int i = 0; i < half_dim; i++) {
+                float c = cos_t[(size_t)pos * half_dim + i];
+                float sn = sin_t[(size_t)pos * half_dim + i];
+                float x0 = p[2 * i];
+                float x1 = p[2 * i + 1];
+                p[2 * i] = x0 * c - x1 * sn;
+                p[2 * i + 1] = x0 * sn + x1 * c;
+            }
+        }
+    }
+    return 0;
 }

@@ -57,6 +57,9 @@ class Oracle:
         L.go_attention_tree.argtypes = [_f32p, _vp, _vp, _vp, _int, _int, _f32p, _f32p, _i32p,
                                         _f32p, _vp, _int, _int, _int, _int, _int, _int, _flt]
         L.go_block_manager_new.restype = _vp
+        L.go_rope_table.argtypes = [_f32p, _f32p, _int, _int, _flt]
+        L.go_rope_apply.argtypes = [_f32p, _int, _int, _int, _int, _f32p, _f32p, _int]
+        L.go_rope_apply.restype = _int
         L.go_block_manager_new.argtypes = [_int, _int]
         L.go_block_manager_delete.argtypes = [_vp]
         L.go_block_manager_allocate.restype = _int
@@ -149,6 +152,23 @@ class Oracle:
         self.lib.go_batched_paged_decode(q, pk, pv, tables, seq_lens, out, _opt(lse), B, Hq, Hkv,
                                          D, block_size, tables.shape[1], scale)
         return out, lse
+
+    def rope_table(self, max_seq_len: int, head_dim: int, theta: float = 10000.0):
+        """(cos, sin), each [max_seq_len, head_dim // 2] float32 (RoPECache::initialize)."""
+        cos = np.zeros((max_seq_len, head_dim // 2), np.float32)
+        sin = np.zeros((max_seq_len, head_dim // 2), np.float32)
+        self.lib.go_rope_table(cos, sin, max_seq_len, head_dim, theta)
+        return cos, sin
+
+    def rope_apply(self, x: np.ndarray, start_pos: int, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+        """Rotated copy of x [seq, heads, D] float32 (RoPECache::apply); raises on its range error."""
+        out = np.ascontiguousarray(x, np.float32).copy()
+        seq, heads, d = out.shape
+        rc = self.lib.go_rope_apply(out, seq, heads, d, start_pos, np.ascontiguousarray(cos),
+                                    np.ascontiguousarray(sin), cos.shape[0])
+        if rc != 0:
+            raise ValueError("RoPE position out of range")
+        return out
 
     def tree_mask(self, parents) -> np.ndarray:
         parents = np.ascontiguousarray(parents, np.int32)
