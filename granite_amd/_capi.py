@@ -116,6 +116,9 @@ class RopeArgs(C.Structure):
         ("freq_base", C.c_float),
         ("write_k_back", C.c_int),
         ("rounding", C.c_int),
+        ("positions", C.c_void_p),
+        ("table_stride", C.c_int64),
+        ("max_blocks_per_seq", C.c_uint32),
     ]
 
 

@@ -34,6 +34,10 @@ struct RopeParams {
     uint16_t* cache_k;  // null: no append
     uint16_t* cache_v;
     const int32_t* table;  // paged pool when set
+    const int32_t* positions;  // per token position (null: start_pos + s)
+    int64_t table_stride;      // entries between the block tables of consecutive tokens (0: one table)
+    uint32_t max_blocks;       // entries of a block table (positions given: rows beyond it are skipped)
+    uint32_t table_positions;  // rows of the cos/sin tables
     const float* cos_t;    // [positions, D/2] or null: evaluate from freq_base
     const float* sin_t;
     uint32_t num_heads_q, num_heads_k, seq_len, head_dim, start_pos;
@@ -69,7 +73,20 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeParams p) {
     const uint64_t idx = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= uint64_t(p.seq_len) * quads) return;
     const uint32_t s = uint32_t(idx / quads), j = uint32_t(idx % quads);
-    const uint32_t pos = p.start_pos + s;
+    // A batch of decode steps gives every token its own position (and block table); a position
+    // comes from device memory then, so what the host checks otherwise is enforced here: no
+    // lookup beyond the tables, no write beyond the cache.
+    uint32_t pos = p.start_pos + s;
+    bool in_range = true;
+    if (p.positions) {
+        const int32_t given = p.positions[s];
+        in_range = given >= 0;
+        pos = in_range ? uint32_t(given) : 0u;
+        if (p.cos_t && pos >= p.table_positions) {
+            in_range = false;
+            pos = 0;
+        }
+    }
 
     float c0, s0, c1, s1;  // of pairs 2j and 2j + 1
     if (p.cos_t) {
@@ -94,8 +111,18 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeParams p) {
     const uint32_t h_all = hq + (p.k ? p.num_heads_k : 0);
     const uint32_t h_end = min(h_begin + kHeadsPerBlock, h_all);
     size_t row = 0;  // cache row of this position (paged: pool row)
-    if (p.cache_k)
-        row = p.table ? size_t(p.table[pos / p.block_size]) * p.block_size + pos % p.block_size : pos;
+    bool store_rows = p.cache_k != nullptr && in_range;
+    if (p.cache_k) {
+        if (p.table) {
+            const uint32_t blk = pos / p.block_size;
+            if (p.positions && blk >= p.max_blocks) store_rows = false;
+            const int32_t* table = p.table + int64_t(s) * p.table_stride;
+            row = size_t(table[store_rows ? blk : 0]) * p.block_size + pos % p.block_size;
+        } else {
+            if (p.positions && pos >= p.max_seq) store_rows = false;
+            row = pos;
+        }
+    }
 
     for (uint32_t h0 = h_begin; h0 < h_end; h0 += 4) {
         float4v x[4], y[4];
@@ -118,7 +145,7 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeParams p) {
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            if (!live[i]) continue;
+            if (!live[i] || !in_range) continue;
             const float2v a = rotate(x[i].x, x[i].y, c0, s0), b = rotate(x[i].z, x[i].w, c1, s1);
             if (!is_k[i]) {
                 *reinterpret_cast<float4v*>(p.q + at[i]) = float4v{a.x, a.y, b.x, b.y};
@@ -131,7 +158,7 @@ __global__ void __launch_bounds__(256) rope_append_kernel(RopeParams p) {
                 continue;
             }
             if (p.write_k_back) *reinterpret_cast<float4v*>(p.k + at[i]) = float4v{a.x, a.y, b.x, b.y};
-            if (p.cache_k) {
+            if (store_rows) {
                 const uint32_t hh = h0 + i - hq;
                 const size_t dst = (p.table ? (row * p.num_heads_k + hh) : (size_t(hh) * p.max_seq + row)) *
                                        p.head_dim + 4 * j;
@@ -164,15 +191,18 @@ int launch_rope_append(const granite_hip_rope_args& a) {
     if (!a.cos_table && !(a.freq_base > 0.0f)) return GRANITE_HIP_EINVAL;
     if (a.rounding != GRANITE_HIP_ROUND_TRUNCATE && a.rounding != GRANITE_HIP_ROUND_NEAREST)
         return GRANITE_HIP_EINVAL;
-    // RoPECache::apply's range check (src/llm/rope.cpp:34-38)
-    if (a.cos_table && uint64_t(a.start_pos) + a.seq_len > a.table_positions) return GRANITE_HIP_EOVERFLOW;
+    // RoPECache::apply's range check (src/llm/rope.cpp:34-38); with per-token positions the
+    // kernel does it per token (a token out of range is left as it is)
+    if (a.cos_table && !a.positions && uint64_t(a.start_pos) + a.seq_len > a.table_positions)
+        return GRANITE_HIP_EOVERFLOW;
     const bool append = a.cache_k != nullptr || a.cache_v != nullptr;
     if (append) {
         if (!a.k || !a.cache_k) return GRANITE_HIP_ENULL;
         if ((a.v == nullptr) != (a.cache_v == nullptr)) return GRANITE_HIP_ENULL;
         if (a.block_table) {
             if (a.block_size == 0) return GRANITE_HIP_EINVAL;
-        } else if (uint64_t(a.start_pos) + a.seq_len > a.max_seq_len) {
+            if (a.positions && a.max_blocks_per_seq == 0) return GRANITE_HIP_EINVAL;
+        } else if (!a.positions && uint64_t(a.start_pos) + a.seq_len > a.max_seq_len) {
             return GRANITE_HIP_EOVERFLOW;
         }
         if (!aligned8(a.cache_k) || (a.cache_v && !aligned8(a.cache_v))) return GRANITE_HIP_EINVAL;
@@ -190,6 +220,10 @@ int launch_rope_append(const granite_hip_rope_args& a) {
     p.cache_k = static_cast<uint16_t*>(a.cache_k);
     p.cache_v = static_cast<uint16_t*>(a.cache_v);
     p.table = append ? a.block_table : nullptr;
+    p.positions = a.positions;
+    p.table_stride = a.positions ? a.table_stride : 0;
+    p.max_blocks = a.max_blocks_per_seq;
+    p.table_positions = a.table_positions;
     p.cos_t = a.cos_table;
     p.sin_t = a.sin_table;
     p.num_heads_q = a.num_heads_q;

@@ -242,7 +242,8 @@ class HipCompute:
     def rope_append(self, *, seq_len, head_dim, start_pos, q=None, num_heads_q=0, q_f16=None, k=None,
                     num_heads_k=0, v=None, cache_k=None, cache_v=None, block_table=None, block_size=0,
                     max_seq_len=0, cos_table=None, sin_table=None, table_positions=0,
-                    freq_base=10000.0, write_k_back=True, rounding=ROUND_TRUNCATE) -> None:
+                    freq_base=10000.0, write_k_back=True, rounding=ROUND_TRUNCATE, positions=None,
+                    table_stride=0, max_blocks_per_seq=0) -> None:
         """Rotation of Q and K and, in the same pass, the append of the rotated K and of V to
         the (contiguous or paged) half cache; with RoPECache's tables the rotation is
         bit-identical to RoPECache::apply (src/llm/rope.cpp:24-92)."""
@@ -252,7 +253,8 @@ class HipCompute:
                      num_heads_q=num_heads_q, num_heads_k=num_heads_k, seq_len=seq_len,
                      head_dim=head_dim, start_pos=start_pos, max_seq_len=max_seq_len,
                      block_size=block_size, freq_base=freq_base, write_k_back=int(write_k_back),
-                     rounding=rounding)
+                     rounding=rounding, positions=_p(positions), table_stride=table_stride,
+                     max_blocks_per_seq=max_blocks_per_seq)
         check(self.lib.granite_hip_rope_append(C.byref(a)), "rope_append")
 
     def build_tree_mask(self, parent_indices, mask_words, num_nodes) -> None:

@@ -4,6 +4,7 @@
 // there with those very values (src/llm/rope.cpp:24-92 is the loop it stands for).
 #pragma once
 
+#include <utility>
 #include <vector>
 
 #include "granite/backend.h"
@@ -32,6 +33,11 @@ public:
     /// [num_kv_heads, max_cache_len, head_dim] at rows start_pos .. (round to nearest).
     Result<void> apply_and_append(Tensor& q, Tensor& k, const Tensor& v, Tensor& cache_k,
                                   Tensor& cache_v, int start_pos, IComputeBackend* backend);
+
+    /// Device copies of the tables on `backend` (made on first use): cos, sin.
+    Result<std::pair<const float*, const float*>> device_tables(IComputeBackend* backend);
+    [[nodiscard]] int max_seq_len() const { return max_seq_len_; }
+    [[nodiscard]] int head_dim() const { return head_dim_; }
 
     [[nodiscard]] const std::vector<float>& cos_cache() const { return cos_; }
     [[nodiscard]] const std::vector<float>& sin_cache() const { return sin_; }

@@ -61,6 +61,17 @@ Result<void> RoPECache::ensure_device_tables(IComputeBackend* backend) {
     return {};
 }
 
+Result<std::pair<const float*, const float*>> RoPECache::device_tables(IComputeBackend* backend) {
+    if (!is_initialized()) return Error(ErrorCode::InvalidState, "RoPE cache not initialized");
+    if (!backend || backend->get_type() != BackendType::HIP)
+        return Error(ErrorCode::BackendNotSupported, "RoPE tables live on the HIP backend only");
+    GRANITE_TRY(ensure_device_tables(backend));
+    const auto* c = static_cast<const float*>(hip_device_pointer(backend, cos_dev_));
+    const auto* s = static_cast<const float*>(hip_device_pointer(backend, sin_dev_));
+    if (!c || !s) return Error(ErrorCode::InternalError, "RoPE tables are not on the device");
+    return std::pair<const float*, const float*>{c, s};
+}
+
 Result<void> RoPECache::apply(Tensor& q, Tensor& k, int start_pos, IComputeBackend* backend) {
     return run(q, k, nullptr, nullptr, nullptr, start_pos, backend);
 }

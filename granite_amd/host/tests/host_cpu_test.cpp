@@ -11,6 +11,7 @@
 #include "granite/hip_compute.h"
 #include "granite/kv_cache.h"
 #include "granite/operators.h"
+#include "granite/paged_batch.h"
 #include "granite/rope.h"
 #include "granite_hip.h"
 #include "host_memory_backend.h"
@@ -539,6 +540,27 @@ TEST_CASE(rope_cache_tables_and_checks) {
     CHECK_CODE(small.apply(half_q, k, 0, &be), ErrorCode::DTypeMismatch);
     // a backend that is not the GPU is refused, never computed on the host
     CHECK_CODE(small.apply(q, k, 0, &be), ErrorCode::BackendNotSupported);
+}
+
+TEST_CASE(paged_decode_batch_checks) {
+    HostMemoryBackend be;
+    REQUIRE(be.initialize().ok());
+    PagedDecodeBatch step;
+    PagedKVPool empty;
+    CHECK_CODE(step.initialize(nullptr, 4, 4, &be), ErrorCode::InvalidState);
+    CHECK_CODE(step.initialize(&empty, 4, 4, &be), ErrorCode::InvalidState);
+    ModelConfig cfg;
+    cfg.num_layers = 1;
+    cfg.num_heads = 4;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = 128;
+    PagedKVPool pool;
+    REQUIRE(pool.initialize(cfg, 2, 64, 16, &be).ok());
+    CHECK_CODE(step.initialize(&pool, 0, 4, &be), ErrorCode::InvalidArgument);
+    // never computed on a backend that is not the GPU
+    CHECK_CODE(step.initialize(&pool, 4, 4, &be), ErrorCode::BackendNotSupported);
+    const int slots[1] = {0};
+    CHECK_CODE(step.begin_step(std::span<const int>(slots, 1)), ErrorCode::InvalidState);
 }
 
 int main(int argc, char** argv) { return hosttest::run_all(argc, argv); }

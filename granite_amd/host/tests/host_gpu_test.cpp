@@ -11,6 +11,7 @@
 #include "granite/hip_compute.h"
 #include "granite/kv_cache.h"
 #include "granite/operators.h"
+#include "granite/paged_batch.h"
 #include "granite/rope.h"
 #include "granite_hip.h"
 
@@ -543,6 +544,180 @@ TEST_CASE(rope_cache_apply_and_append) {
             }
     CHECK(wrong == 0);
     CHECK_CODE(rope.apply_and_append(Q2, K2, V, CK, CV, 270, backend()), ErrorCode::InvalidArgument);
+}
+
+TEST_CASE(paged_prefill_then_batched_decode_steps) {
+    REQUIRE(backend() != nullptr);
+    HipCompute* hc = get_hip_compute();
+    REQUIRE(hc != nullptr);
+    ModelConfig cfg;
+    cfg.num_layers = 2;
+    cfg.num_heads = 8;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = D;
+    const int bs = 16, hq = 8, hkv = 2, max_blocks = 12, max_pos = max_blocks * bs;
+    PagedKVPool pool;
+    REQUIRE(pool.initialize(cfg, 5, 26 * bs, bs, backend()).ok());  // 26 blocks in all
+    BlockManager& mgr = pool.block_manager();
+    RoPECache rope;
+    rope.initialize(max_pos, D, 10000.0f);
+    std::vector<float> cos_t(size_t(max_pos) * D / 2), sin_t(cos_t.size());
+    go_rope_table(cos_t.data(), sin_t.data(), max_pos, D, 10000.0f);
+    auto rope_tables = rope.device_tables(backend());
+    REQUIRE(rope_tables.ok());
+    const float scale = 1.0f / std::sqrt(float(D));
+
+    // the oracle's pools start from the device's bytes
+    std::vector<std::vector<uint16_t>> want_k, want_v;
+    for (int l = 0; l < 2; ++l) {
+        want_k.push_back(download<uint16_t>(mgr.k_cache(l)));
+        want_v.push_back(download<uint16_t>(mgr.v_cache(l)));
+    }
+
+    // ---- paged prefill: every sequence's prompt in one rotate-and-append launch per layer
+    // (the reference fills a paged cache one token at a time,
+    // tools/benchmark_paged_attention.mm:348-363)
+    const int batch = 4;
+    const int prompt[batch] = {37, 1, 150, 64};
+    int slots[batch];
+    uint32_t seed = 7000;
+    for (int b = 0; b < batch; ++b) {
+        slots[b] = pool.acquire_slot();
+        REQUIRE(slots[b] >= 0);
+        PagedKVCache& seq = pool.get_cache(slots[b]);
+        REQUIRE(seq.append_tokens(prompt[b]));
+        std::vector<int32_t> table(seq.block_table().begin(), seq.block_table().end());
+        Tensor T = upload({int64_t(table.size())}, DataType::INT32, table);
+        for (int l = 0; l < 2; ++l) {
+            auto k = randn(size_t(prompt[b]) * hkv * D, seed++), v = randn(size_t(prompt[b]) * hkv * D, seed++);
+            Tensor K = upload({prompt[b], hkv, D}, DataType::FP32, k);
+            Tensor V = upload({prompt[b], hkv, D}, DataType::FP32, v);
+            granite_hip_rope_args r{};
+            r.k = hip_device_pointer(backend(), K.buffer());
+            r.v = hip_device_pointer(backend(), V.buffer());
+            r.cache_k = hip_device_pointer(backend(), mgr.k_cache(l).buffer());
+            r.cache_v = hip_device_pointer(backend(), mgr.v_cache(l).buffer());
+            r.block_table = static_cast<const int32_t*>(hip_device_pointer(backend(), T.buffer()));
+            r.block_size = bs;
+            r.num_heads_k = hkv;
+            r.seq_len = uint32_t(prompt[b]);
+            r.head_dim = D;
+            r.start_pos = 0;
+            r.cos_table = rope_tables.value().first;
+            r.sin_table = rope_tables.value().second;
+            r.table_positions = max_pos;
+            r.rounding = GRANITE_HIP_ROUND_TRUNCATE;
+            CHECK_OK(hc->rope_append(r));
+            hc->sync();
+            // oracle: rotate, then the paged append on [Hkv, new_len, D]
+            CHECK(go_rope_apply(k.data(), prompt[b], hkv, D, 0, cos_t.data(), sin_t.data(), max_pos) == 0);
+            std::vector<float> kt(k.size()), vt(v.size());
+            for (int s = 0; s < prompt[b]; ++s)
+                for (int h = 0; h < hkv; ++h)
+                    for (int d = 0; d < D; ++d) {
+                        kt[(size_t(h) * prompt[b] + s) * D + d] = k[(size_t(s) * hkv + h) * D + d];
+                        vt[(size_t(h) * prompt[b] + s) * D + d] = v[(size_t(s) * hkv + h) * D + d];
+                    }
+            go_paged_kv_cache_append_f32(want_k[l].data(), kt.data(), table.data(), hkv, D, 0, prompt[b], bs);
+            go_paged_kv_cache_append_f32(want_v[l].data(), vt.data(), table.data(), hkv, D, 0, prompt[b], bs);
+            backend()->destroy_buffer(K.buffer());
+            backend()->destroy_buffer(V.buffer());
+        }
+        backend()->destroy_buffer(T.buffer());
+    }
+    for (int l = 0; l < 2; ++l) {
+        CHECK(download<uint16_t>(mgr.k_cache(l)) == want_k[l]);  // bit exact
+        CHECK(download<uint16_t>(mgr.v_cache(l)) == want_v[l]);
+    }
+
+    // ---- batched decode steps
+    PagedDecodeBatch step;
+    CHECK_CODE(step.begin_step(std::span<const int>(slots, batch)), ErrorCode::InvalidState);
+    REQUIRE(step.initialize(&pool, 8, max_blocks, backend()).ok());
+    step.set_rounding(GRANITE_HIP_ROUND_TRUNCATE);
+    Tensor Qbad = Tensor::allocate({batch, hq, D}, DataType::FP32, backend()).take();
+    CHECK_CODE(step.run_layer(0, Qbad, Qbad, Qbad, Qbad, scale, &rope), ErrorCode::InvalidState);
+    int lens[batch];
+    for (int b = 0; b < batch; ++b) lens[b] = prompt[b];
+    for (int it = 0; it < 3; ++it) {
+        auto failed = step.begin_step(std::span<const int>(slots, batch));
+        REQUIRE(failed.ok());
+        CHECK(failed.value().empty());
+        CHECK(step.batch_size() == batch);
+        std::vector<int32_t> tables(size_t(batch) * max_blocks, 0), seq_lens(batch);
+        for (int b = 0; b < batch; ++b) {
+            lens[b] += 1;
+            CHECK(pool.get_cache(slots[b]).seq_len() == lens[b]);
+            CHECK(step.seq_lens()[b] == lens[b]);
+            seq_lens[b] = lens[b];
+            const auto& t = pool.get_cache(slots[b]).block_table();
+            std::copy(t.begin(), t.end(), tables.begin() + size_t(b) * max_blocks);
+        }
+        for (int l = 0; l < 2; ++l) {
+            auto q = randn(size_t(batch) * hq * D, seed++), k = randn(size_t(batch) * hkv * D, seed++),
+                 v = randn(size_t(batch) * hkv * D, seed++);
+            Tensor Q = upload({batch, hq, D}, DataType::FP32, q);
+            Tensor K = upload({batch, hkv, D}, DataType::FP32, k);
+            Tensor V = upload({batch, hkv, D}, DataType::FP32, v);
+            Tensor O = Tensor::allocate({batch, hq, D}, DataType::FP32, backend()).take();
+            CHECK_OK(step.run_layer(l, Q, K, V, O, scale, &rope));
+            // oracle: sequence by sequence, as the reference's loop would
+            for (int b = 0; b < batch; ++b) {
+                const int pos = lens[b] - 1;
+                CHECK(go_rope_apply(q.data() + size_t(b) * hq * D, 1, hq, D, pos, cos_t.data(), sin_t.data(), max_pos) == 0);
+                CHECK(go_rope_apply(k.data() + size_t(b) * hkv * D, 1, hkv, D, pos, cos_t.data(), sin_t.data(), max_pos) == 0);
+                go_paged_kv_cache_append_f32(want_k[l].data(), k.data() + size_t(b) * hkv * D,
+                                             tables.data() + size_t(b) * max_blocks, hkv, D, pos, 1, bs);
+                go_paged_kv_cache_append_f32(want_v[l].data(), v.data() + size_t(b) * hkv * D,
+                                             tables.data() + size_t(b) * max_blocks, hkv, D, pos, 1, bs);
+            }
+            std::vector<float> want(q.size());
+            go_batched_paged_decode(q.data(), want_k[l].data(), want_v[l].data(), tables.data(), seq_lens.data(),
+                                    want.data(), nullptr, batch, hq, hkv, D, bs, max_blocks, scale);
+            CHECK(download<float>(Q) == q);                           // rotated Q and K: the oracle's bits
+            CHECK(download<float>(K) == k);
+            CHECK(download<uint16_t>(mgr.k_cache(l)) == want_k[l]);   // pools bit exact
+            CHECK(download<uint16_t>(mgr.v_cache(l)) == want_v[l]);
+            CHECK(close_enough(download<float>(O), want, "batched decode step"));
+            for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+        }
+    }
+
+    // ---- a sequence that cannot take a token: reported, left out, the others go on
+    // 37+3, 1+3, 150+3, 64+3 tokens hold 3 + 1 + 10 + 5 = 19 of 26 blocks; a fifth sequence takes the rest
+    int extra = pool.acquire_slot();
+    REQUIRE(extra >= 0);
+    REQUIRE(pool.get_cache(extra).append_tokens(7 * bs));
+    CHECK(pool.num_free_blocks() == 0);
+    // sequence 3 is at 67 tokens: 5 blocks hold 80, so it still fits; sequence 2 at 153 of 160 too;
+    // push sequence 0 (40 tokens, 3 blocks = 48) to its block edge to make it need a new block
+    REQUIRE(pool.get_cache(slots[0]).append_tokens(8));
+    lens[0] += 8;
+    {
+        auto failed = step.begin_step(std::span<const int>(slots, batch));
+        REQUIRE(failed.ok());
+        REQUIRE(failed.value().size() == 1);
+        CHECK(failed.value()[0] == slots[0]);
+        CHECK(step.seq_lens()[0] == 0);
+        CHECK(pool.get_cache(slots[0]).seq_len() == lens[0]);  // unchanged
+        auto q = randn(size_t(batch) * hq * D, seed++), k = randn(size_t(batch) * hkv * D, seed++),
+             v = randn(size_t(batch) * hkv * D, seed++);
+        Tensor Q = upload({batch, hq, D}, DataType::FP32, q);
+        Tensor K = upload({batch, hkv, D}, DataType::FP32, k);
+        Tensor V = upload({batch, hkv, D}, DataType::FP32, v);
+        std::vector<float> sentinel(q.size(), -7.0f);
+        Tensor O = upload({batch, hq, D}, DataType::FP32, sentinel);
+        CHECK_OK(step.run_layer(0, Q, K, V, O, scale, &rope));
+        auto got_q = download<float>(Q), got_o = download<float>(O);
+        bool untouched = true;
+        for (size_t i = 0; i < size_t(hq) * D; ++i) untouched = untouched && got_q[i] == q[i] && got_o[i] == -7.0f;
+        CHECK(untouched);                                  // row 0: neither rotated nor written
+        bool others_written = true;
+        for (size_t i = size_t(hq) * D; i < got_o.size(); ++i) others_written = others_written && got_o[i] != -7.0f;
+        CHECK(others_written);
+        CHECK(download<uint16_t>(mgr.k_cache(1)) == want_k[1]);  // the other layer's pool is not touched
+    }
+    CHECK_CODE(step.begin_step(std::span<const int>(slots, 0)), ErrorCode::InvalidArgument);
 }
 
 int main(int argc, char** argv) {

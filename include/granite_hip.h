@@ -326,7 +326,16 @@ int granite_hip_rope_multihead(void *q, void *k, uint32_t num_heads_q, uint32_t 
  *                 + seq_len > table_positions -> GRANITE_HIP_EOVERFLOW, its
  *                 range check (rope.cpp:34-38).  Both NULL: evaluated from
  *                 freq_base on the device.
- *   rounding      float -> half conversion of the cache rows */
+ *   rounding      float -> half conversion of the cache rows
+ *   positions     NULL, or device int32[seq_len]: the position of every token
+ *                 (a batch of decode steps: token s belongs to sequence s).
+ *                 block_table then advances by table_stride entries per token
+ *                 (0: one table) and holds max_blocks_per_seq entries per
+ *                 sequence.  The host cannot check values that live on the
+ *                 device, so the kernel does: a token whose position is
+ *                 negative or beyond the cos/sin tables is left untouched, one
+ *                 whose position is beyond its cache (max_seq_len, or
+ *                 max_blocks_per_seq blocks) is rotated but not stored. */
 typedef struct granite_hip_rope_args {
     void *q;
     void *q_f16;
@@ -344,6 +353,9 @@ typedef struct granite_hip_rope_args {
     float freq_base;
     int write_k_back;
     int rounding;
+    const int32_t *positions;
+    int64_t table_stride;
+    uint32_t max_blocks_per_seq;
 } granite_hip_rope_args;
 
 int granite_hip_rope_append(const granite_hip_rope_args *args);

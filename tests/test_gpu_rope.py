@@ -143,6 +143,50 @@ def test_rope_full_chunk_shape_round_trip(gpu, oracle):
     assert np.abs(dq.read(np.float32, q.shape) - q).max() <= 1e-6
 
 
+def test_rope_append_batched_decode_positions(gpu, oracle):
+    """A batch of decode steps: token s belongs to sequence s, at its own position and with its
+    own block table.  Bit-exact against the oracle sequence by sequence; tokens whose position
+    is negative or beyond the cos/sin tables are left alone, one beyond its block table is
+    rotated but not stored."""
+    B, hq, hkv, d, bs, max_blocks, positions_max = 6, 8, 2, 128, 16, 4, 100
+    rng = np.random.default_rng(77)
+    pos = np.array([0, 17, 63, -1, 100, 70], np.int32)   # 3: negative, 4: beyond the tables, 5: beyond 4 blocks
+    q = rng.standard_normal((B, hq, d)).astype(np.float32)
+    k = rng.standard_normal((B, hkv, d)).astype(np.float32)
+    v = rng.standard_normal((B, hkv, d)).astype(np.float32)
+    cos, sin = oracle.rope_table(positions_max, d, 10000.0)
+    nblk = B * max_blocks
+    tables = rng.permutation(nblk).astype(np.int32).reshape(B, max_blocks)
+    pool_k = np.full((nblk * bs, hkv, d), SENT, np.uint16)
+    pool_v = np.full((nblk * bs, hkv, d), SENT + 1, np.uint16)
+    want_q, want_k, want_pk, want_pv = q.copy(), k.copy(), pool_k.copy(), pool_v.copy()
+    for b in range(B):
+        p = int(pos[b])
+        if p < 0 or p >= positions_max:
+            continue
+        want_q[b:b + 1] = oracle.rope_apply(q[b:b + 1], p, cos, sin)
+        want_k[b:b + 1] = oracle.rope_apply(k[b:b + 1], p, cos, sin)
+        if p // bs < max_blocks:
+            row = tables[b, p // bs] * bs + p % bs
+            want_pk[row] = oracle.fp32_to_fp16(want_k[b])
+            want_pv[row] = oracle.fp32_to_fp16(v[b])
+    dq, dk, dv, dpk, dpv = dev(q), dev(k), dev(v), dev(pool_k), dev(pool_v)
+    dcos, dsin, dt, dpos = dev(cos), dev(sin), dev(tables), dev(pos)
+    gpu.rope_append(seq_len=B, head_dim=d, start_pos=0, q=dq, num_heads_q=hq, k=dk, num_heads_k=hkv, v=dv,
+                    cache_k=dpk, cache_v=dpv, block_table=dt, block_size=bs, cos_table=dcos, sin_table=dsin,
+                    table_positions=positions_max, positions=dpos, table_stride=max_blocks,
+                    max_blocks_per_seq=max_blocks, rounding=ROUND_TRUNCATE)
+    gpu.sync()
+    assert np.array_equal(dq.read(np.float32, q.shape), want_q)
+    assert np.array_equal(dk.read(np.float32, k.shape), want_k)
+    assert np.array_equal(dpk.read(np.uint16, pool_k.shape), want_pk)
+    assert np.array_equal(dpv.read(np.uint16, pool_v.shape), want_pv)
+    with pytest.raises(GraniteHipError) as e:   # per-token positions over a paged cache need the table length
+        gpu.rope_append(seq_len=B, head_dim=d, start_pos=0, k=dk, num_heads_k=hkv, v=dv, cache_k=dpk,
+                        cache_v=dpv, block_table=dt, block_size=bs, positions=dpos, table_stride=max_blocks)
+    assert e.value.code == _capi.EINVAL
+
+
 def test_rope_argument_errors(gpu):
     buf = dev(np.zeros(4096, np.float32))
     base = dict(seq_len=2, head_dim=128, start_pos=0, q=buf, num_heads_q=2, k=buf, num_heads_k=1)
