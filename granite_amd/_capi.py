@@ -169,6 +169,8 @@ SIGNATURES = {
     "granite_hip_decode_attention": (_int, [C.POINTER(DecodeArgs)]),
     "granite_hip_attention": (_int, [C.POINTER(AttentionArgs)]),
     "granite_hip_build_tree_mask": (_int, [_vp, _vp, _u32]),
+    "granite_hip_kv_commit_accepted": (_int, [_vp, _vp, _int, _i64, _i64, _u32, _vp, _u32, _vp, _vp, _vp, _u32,
+                                             _u32, _u32, _u32, _u32, _int]),
     "granite_hip_rope_multihead": (_int, [_vp, _vp, _u32, _u32, _u32, _u32, _u32, _f32]),
     "granite_hip_rope_append": (_int, [C.POINTER(RopeArgs)]),
     "granite_hip_workspace_bytes": (C.c_size_t, []),

@@ -297,6 +297,27 @@ int granite_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
     return GRANITE_HIP_OK;
 }
 
+int granite_hip_kv_commit_accepted(const void* k_tree, const void* v_tree, int src_dtype,
+                                   int64_t src_tok_stride, int64_t src_head_stride,
+                                   uint32_t num_nodes, const int32_t* accepted_nodes,
+                                   uint32_t num_accepted, void* k_cache, void* v_cache,
+                                   const int32_t* block_table, uint32_t num_kv_heads,
+                                   uint32_t head_dim, uint32_t start_pos, uint32_t block_size,
+                                   uint32_t max_seq_len, int rounding) {
+    GHIP_REQUIRE_INIT();
+    if (num_accepted == 0) return GRANITE_HIP_OK;
+    if (!accepted_nodes) return GRANITE_HIP_ENULL;
+    if (num_nodes == 0) return GRANITE_HIP_EINVAL;
+    if (block_table)
+        return ghip::launch_kv_append_paged(k_tree, v_tree, src_dtype, src_tok_stride, src_head_stride,
+                                            k_cache, v_cache, block_table, num_kv_heads, head_dim,
+                                            start_pos, num_accepted, block_size, rounding,
+                                            accepted_nodes, num_nodes);
+    return ghip::launch_kv_append_contig(k_cache, v_cache, k_tree, v_tree, src_dtype, src_tok_stride,
+                                         src_head_stride, num_kv_heads, head_dim, start_pos,
+                                         num_accepted, max_seq_len, rounding, accepted_nodes, num_nodes);
+}
+
 // ---- RoPE (+ append) -----------------------------------------------------
 
 int granite_hip_rope_append(const granite_hip_rope_args* args) {

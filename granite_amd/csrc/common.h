@@ -64,12 +64,14 @@ inline int launch_status() {
 int launch_kv_append_contig(void* cache_k, void* cache_v, const void* new_k, const void* new_v,
                             int src_dtype, int64_t src_tok_stride, int64_t src_head_stride,
                             uint32_t num_kv_heads, uint32_t head_dim, uint32_t current_len,
-                            uint32_t new_len, uint32_t max_seq_len, int rounding);
+                            uint32_t new_len, uint32_t max_seq_len, int rounding,
+                            const int32_t* src_index = nullptr, uint32_t src_tokens = 0);
 int launch_kv_append_paged(const void* new_k, const void* new_v, int src_dtype,
                            int64_t src_tok_stride, int64_t src_head_stride, void* k_cache,
                            void* v_cache, const int32_t* block_table, uint32_t num_kv_heads,
                            uint32_t head_dim, uint32_t start_pos, uint32_t new_len,
-                           uint32_t block_size, int rounding);
+                           uint32_t block_size, int rounding, const int32_t* src_index = nullptr,
+                           uint32_t src_tokens = 0);
 int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const void* v_cache,
                            const int32_t* block_table, uint32_t num_kv_heads, uint32_t head_dim,
                            uint32_t len, uint32_t block_size, uint32_t max_seq_len);

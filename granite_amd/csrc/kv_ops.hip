@@ -60,6 +60,9 @@ struct AppendParams {
     const void* src[2];
     uint16_t* dst[2];
     const int32_t* table;  // nullptr: contiguous cache
+    const int32_t* src_index;  // nullptr, or: new token s is source token src_index[s] (out of
+                               // [0, src_tokens): the token is skipped)
+    uint32_t src_tokens;
     int64_t src_tok_stride, src_head_stride;
     uint32_t num_kv_heads, head_dim, first_pos, new_len;
     uint32_t max_seq;     // contiguous
@@ -94,7 +97,13 @@ __global__ void __launch_bounds__(256) kv_append_vec_kernel(AppendParams p) {
             s = rest % p.new_len;
             h = rest / p.new_len;
         }
-        const SrcT* sp = src + int64_t(s) * p.src_tok_stride + int64_t(h) * p.src_head_stride +
+        uint32_t s_src = s;
+        if (p.src_index) {
+            const int32_t picked = p.src_index[s];
+            if (picked < 0 || uint32_t(picked) >= p.src_tokens) continue;
+            s_src = uint32_t(picked);
+        }
+        const SrcT* sp = src + int64_t(s_src) * p.src_tok_stride + int64_t(h) * p.src_head_stride +
                          v * kVec;
         uint4v val = load8_as_half<SrcT, kNearest>(sp);
         *reinterpret_cast<uint4v*>(dst + dst_row_offset(p, p.first_pos + s, h) + v * kVec) = val;
@@ -115,7 +124,13 @@ __global__ void __launch_bounds__(256) kv_append_scalar_kernel(AppendParams p) {
         uint32_t rest = i / p.head_dim;
         uint32_t h = rest % p.num_kv_heads;
         uint32_t s = rest / p.num_kv_heads;
-        SrcT x = src[int64_t(s) * p.src_tok_stride + int64_t(h) * p.src_head_stride + d];
+        uint32_t s_src = s;
+        if (p.src_index) {
+            const int32_t picked = p.src_index[s];
+            if (picked < 0 || uint32_t(picked) >= p.src_tokens) continue;
+            s_src = uint32_t(picked);
+        }
+        SrcT x = src[int64_t(s_src) * p.src_tok_stride + int64_t(h) * p.src_head_stride + d];
         uint16_t hbits;
         if constexpr (sizeof(SrcT) == 2) {
             hbits = x;
@@ -199,9 +214,12 @@ int launch_append(const AppendParams& p, int src_dtype, int rounding) {
 int launch_kv_append_contig(void* cache_k, void* cache_v, const void* new_k, const void* new_v,
                             int src_dtype, int64_t src_tok_stride, int64_t src_head_stride,
                             uint32_t num_kv_heads, uint32_t head_dim, uint32_t current_len,
-                            uint32_t new_len, uint32_t max_seq_len, int rounding) {
+                            uint32_t new_len, uint32_t max_seq_len, int rounding,
+                            const int32_t* src_index, uint32_t src_tokens) {
     if (uint64_t(current_len) + new_len > max_seq_len) return GRANITE_HIP_EOVERFLOW;
     AppendParams p{};
+    p.src_index = src_index;
+    p.src_tokens = src_tokens;
     p.src[0] = new_k;
     p.src[1] = new_v;
     p.dst[0] = static_cast<uint16_t*>(cache_k);
@@ -222,10 +240,13 @@ int launch_kv_append_paged(const void* new_k, const void* new_v, int src_dtype,
                            int64_t src_tok_stride, int64_t src_head_stride, void* k_cache,
                            void* v_cache, const int32_t* block_table, uint32_t num_kv_heads,
                            uint32_t head_dim, uint32_t start_pos, uint32_t new_len,
-                           uint32_t block_size, int rounding) {
+                           uint32_t block_size, int rounding, const int32_t* src_index,
+                           uint32_t src_tokens) {
     if (!block_table) return GRANITE_HIP_ENULL;
     if (block_size == 0) return GRANITE_HIP_EINVAL;
     AppendParams p{};
+    p.src_index = src_index;
+    p.src_tokens = src_tokens;
     p.src[0] = new_k;
     p.src[1] = new_v;
     p.dst[0] = static_cast<uint16_t*>(k_cache);

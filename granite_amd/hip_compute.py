@@ -232,6 +232,17 @@ class HipCompute:
                           num_kv_heads=num_kv_heads, head_dim=head_dim, scale=scale)
         check(self.lib.granite_hip_attention(C.byref(a)), "attention")
 
+    def kv_commit_accepted(self, k_tree, v_tree, src_dtype, src_tok_stride, src_head_stride, num_nodes,
+                           accepted_nodes, num_accepted, k_cache, v_cache, num_kv_heads, head_dim,
+                           start_pos, block_table=None, block_size=0, max_seq_len=0,
+                           rounding=ROUND_TRUNCATE) -> None:
+        """Writes the accepted tree nodes' K/V rows, in path order, to cache positions
+        start_pos .. (the step src/llm/speculative_runner.cpp:871-882 presumes done)."""
+        check(self.lib.granite_hip_kv_commit_accepted(
+            _p(k_tree), _p(v_tree), src_dtype, src_tok_stride, src_head_stride, num_nodes,
+            _p(accepted_nodes), num_accepted, _p(k_cache), _p(v_cache), _p(block_table), num_kv_heads,
+            head_dim, start_pos, block_size, max_seq_len, rounding), "kv_commit_accepted")
+
     def rope_multihead(self, q, k, num_heads_q, num_heads_k, seq_len, head_dim, start_pos,
                        freq_base=10000.0) -> None:
         """MetalCompute::rope_multihead (include/granite/metal_compute.h:728-739): q

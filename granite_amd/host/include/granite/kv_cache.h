@@ -13,6 +13,7 @@
 
 #include <cstdint>
 #include <utility>
+#include <span>
 #include <vector>
 
 #include "granite/tensor.h"
@@ -194,9 +195,25 @@ class SpeculationTree {
     // Longest root path whose tokens equal target_choices position by position;
     // at the first mismatch the target's own token closes the path.
     std::vector<int32_t> find_accepted_path(const std::vector<int32_t>& target_choices) const;
+    // The node indices of that path's tree nodes, root first (the closing token of a
+    // mismatch is the target's own and has no node).  Not in the reference: it is what the
+    // commit below needs.
+    std::vector<int> find_accepted_nodes(const std::vector<int32_t>& target_choices) const;
 
   private:
     std::vector<Node> nodes_;
 };
+
+// Commit of an accepted path into a sequence's paged cache: the sequence is brought to
+// original_len + accepted_nodes.size() tokens (blocks past that are freed, as the runner's
+// truncate does, src/llm/speculative_runner.cpp:871-882; missing ones are allocated) and, for
+// every layer, rows original_len .. receive the K/V of the accepted tree nodes in path order
+// out of k_tree[layer] / v_tree[layer] ([num_kv_heads, num_nodes, head_dim] FP16).  The
+// reference's runner presumes those rows are already in the cache, yet nothing on its tree
+// path writes them: the semantics here are this build's.
+[[nodiscard]] Result<void> commit_tree_path(PagedKVCache& sequence, int original_len,
+                                            std::span<const int> accepted_nodes,
+                                            std::span<const Tensor> k_tree,
+                                            std::span<const Tensor> v_tree, IComputeBackend* backend);
 
 }  // namespace granite

@@ -7,6 +7,7 @@
 
 #include "granite/hip_backend.h"
 #include "granite/hip_compute.h"
+#include "granite_hip.h"
 
 namespace granite {
 
@@ -242,6 +243,73 @@ int PagedKVPool::num_free_slots() const {
     int n = 0;
     for (bool used : in_use_) n += used ? 0 : 1;
     return n;
+}
+
+Result<void> commit_tree_path(PagedKVCache& sequence, int original_len,
+                              std::span<const int> accepted_nodes, std::span<const Tensor> k_tree,
+                              std::span<const Tensor> v_tree, IComputeBackend* backend) {
+    BlockManager* blocks = sequence.block_manager();
+    if (!blocks || !blocks->is_initialized())
+        return Error(ErrorCode::InvalidState, "Sequence has no block manager");
+    const PagedKVConfig& cfg = blocks->config();
+    if (original_len < 0 || static_cast<int>(k_tree.size()) != cfg.num_layers ||
+        v_tree.size() != k_tree.size())
+        return Error(ErrorCode::InvalidArgument, "One K and one V tree tensor per layer");
+    if (!backend || backend->get_type() != BackendType::HIP)
+        return Error(ErrorCode::BackendNotSupported, "commit_tree_path runs on the HIP backend only");
+    int64_t num_nodes = 0;
+    for (size_t l = 0; l < k_tree.size(); ++l) {
+        const Tensor &k = k_tree[l], &v = v_tree[l];
+        if (k.ndim() != 3 || v.ndim() != 3 || k.size(0) != cfg.num_kv_heads || k.size(2) != cfg.head_dim ||
+            v.size(0) != k.size(0) || v.size(1) != k.size(1) || v.size(2) != k.size(2) ||
+            (l > 0 && k.size(1) != num_nodes))
+            return Error(ErrorCode::ShapeMismatch, "Tree K/V are [num_kv_heads, num_nodes, head_dim]");
+        if (k.dtype() != DataType::FP16 || v.dtype() != DataType::FP16)
+            return Error(ErrorCode::DTypeMismatch, "Tree K/V rows are FP16");
+        num_nodes = k.size(1);
+    }
+    const int n = static_cast<int>(accepted_nodes.size());
+    for (int node : accepted_nodes)
+        if (node < 0 || node >= num_nodes) return Error(ErrorCode::InvalidArgument, "Accepted node outside the tree");
+    const int target_len = original_len + n;
+    if (sequence.seq_len() > target_len) {
+        sequence.truncate(target_len);
+    } else if (sequence.seq_len() < target_len && !sequence.append_tokens(target_len - sequence.seq_len())) {
+        return Error(ErrorCode::AllocationFailed, "No free blocks for the accepted tokens");
+    }
+    if (n == 0) return {};
+
+    std::vector<int32_t> nodes32(accepted_nodes.begin(), accepted_nodes.end());
+    std::vector<int32_t> table(sequence.block_table().begin(), sequence.block_table().end());
+    GRANITE_TRY_ASSIGN(d_nodes, backend->create_buffer_from_host(nodes32.data(), BufferDesc::device(nodes32.size() * 4)));
+    auto made = backend->create_buffer_from_host(table.data(), BufferDesc::device(table.size() * 4));
+    if (!made.ok()) {
+        backend->destroy_buffer(d_nodes);
+        return made.error();
+    }
+    const BufferHandle d_table = made.value();
+    auto ptr = [&](const Tensor& t) -> char* {
+        auto* p = static_cast<char*>(hip_device_pointer(backend, t.buffer()));
+        return p ? p + t.buffer_offset() : nullptr;
+    };
+    Result<void> status;
+    for (int l = 0; l < cfg.num_layers && status.ok(); ++l) {
+        status = hip_status_to_result(
+            granite_hip_kv_commit_accepted(
+                ptr(k_tree[l]), ptr(v_tree[l]), GRANITE_HIP_F16, cfg.head_dim, num_nodes * cfg.head_dim,
+                static_cast<uint32_t>(num_nodes),
+                static_cast<const int32_t*>(hip_device_pointer(backend, d_nodes)), static_cast<uint32_t>(n),
+                ptr(blocks->k_cache(l)), ptr(blocks->v_cache(l)),
+                static_cast<const int32_t*>(hip_device_pointer(backend, d_table)),
+                static_cast<uint32_t>(cfg.num_kv_heads), static_cast<uint32_t>(cfg.head_dim),
+                static_cast<uint32_t>(original_len), static_cast<uint32_t>(blocks->block_size()), 0,
+                GRANITE_HIP_ROUND_TRUNCATE),
+            "granite_hip_kv_commit_accepted");
+    }
+    (void)backend->wait_for_completion();  // the two small buffers are released below
+    backend->destroy_buffer(d_nodes);
+    backend->destroy_buffer(d_table);
+    return status;
 }
 
 }  // namespace granite

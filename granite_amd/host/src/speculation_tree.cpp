@@ -92,4 +92,29 @@ std::vector<int32_t> SpeculationTree::find_accepted_path(
     return best;
 }
 
+std::vector<int> SpeculationTree::find_accepted_nodes(const std::vector<int32_t>& target_choices) const {
+    // Replays the accepted token path from the root: position i of the path is the child of
+    // the previous node whose token the target chose.
+    std::vector<int> nodes;
+    const std::vector<int32_t> tokens = find_accepted_path(target_choices);
+    if (nodes_.empty() || tokens.empty()) return nodes;
+    int cur = 0;
+    for (size_t i = 0; i < tokens.size(); ++i) {
+        if (i == 0) {
+            if (nodes_[0].token != tokens[0]) break;  // the root itself was replaced
+        } else {
+            int next = -1;
+            for (int child : nodes_[cur].children)
+                if (nodes_[child].token == tokens[i]) {
+                    next = child;
+                    break;
+                }
+            if (next < 0) break;  // the closing token of a mismatch: no node
+            cur = next;
+        }
+        nodes.push_back(cur);
+    }
+    return nodes;
+}
+
 }  // namespace granite

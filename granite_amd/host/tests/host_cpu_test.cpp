@@ -485,6 +485,12 @@ TEST_CASE(speculation_tree) {
     CHECK((tree.find_accepted_path({7, 11}) == P{7}));                      // root mismatch
     CHECK((tree.find_accepted_path({10}) == P{10}));
     CHECK((tree.find_accepted_path({10, 11}) == P{10, 11}));
+    using N = std::vector<int>;
+    CHECK((tree.find_accepted_nodes({10, 11, 14, 16}) == N{0, 1, 4, 6}));
+    CHECK((tree.find_accepted_nodes({10, 12, 15, 99}) == N{0, 2, 5}));
+    CHECK((tree.find_accepted_nodes({10, 11, 99, 5}) == N{0, 1}));   // the closing token has no node
+    CHECK(tree.find_accepted_nodes({7, 11}).empty());                 // the root was replaced
+    CHECK((tree.find_accepted_nodes({10}) == N{0}));
     tree.clear();
     CHECK(tree.size() == 0 && tree.max_depth() == 0);
 }
@@ -540,6 +546,28 @@ TEST_CASE(rope_cache_tables_and_checks) {
     CHECK_CODE(small.apply(half_q, k, 0, &be), ErrorCode::DTypeMismatch);
     // a backend that is not the GPU is refused, never computed on the host
     CHECK_CODE(small.apply(q, k, 0, &be), ErrorCode::BackendNotSupported);
+}
+
+TEST_CASE(commit_tree_path_checks) {
+    HostMemoryBackend be;
+    REQUIRE(be.initialize().ok());
+    PagedKVConfig cfg;
+    cfg.block_size = 16;
+    cfg.num_blocks = 8;
+    cfg.num_layers = 1;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = 128;
+    BlockManager mgr;
+    REQUIRE(mgr.initialize(cfg, &be).ok());
+    PagedKVCache seq(&mgr);
+    PagedKVCache orphan;
+    Tensor kt = Tensor::allocate({2, 6, 128}, DataType::FP16, &be).take();
+    std::vector<Tensor> trees{kt};
+    const int nodes[2] = {0, 3}, bad_nodes[1] = {6};
+    CHECK_CODE(commit_tree_path(orphan, 0, nodes, trees, trees, &be), ErrorCode::InvalidState);
+    CHECK_CODE(commit_tree_path(seq, 0, nodes, {}, {}, &be), ErrorCode::InvalidArgument);
+    CHECK_CODE(commit_tree_path(seq, 0, nodes, trees, trees, &be), ErrorCode::BackendNotSupported);
+    (void)bad_nodes;
 }
 
 TEST_CASE(paged_decode_batch_checks) {

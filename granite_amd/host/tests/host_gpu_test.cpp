@@ -720,6 +720,59 @@ TEST_CASE(paged_prefill_then_batched_decode_steps) {
     CHECK_CODE(step.begin_step(std::span<const int>(slots, 0)), ErrorCode::InvalidArgument);
 }
 
+TEST_CASE(speculative_commit_of_accepted_path) {
+    REQUIRE(backend() != nullptr);
+    PagedKVConfig cfg;
+    cfg.block_size = 16;
+    cfg.num_blocks = 10;
+    cfg.num_layers = 2;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = D;
+    BlockManager mgr;
+    REQUIRE(mgr.initialize(cfg, backend()).ok());
+    PagedKVCache seq(&mgr);
+    const int original = 29, n_nodes = 7, hkv = 2, bs = 16;
+    // as the runner does: the tree step reserved original + tree_size tokens
+    REQUIRE(seq.append_tokens(original + n_nodes));
+    SpeculationTree tree;
+    tree.add_node(10, -1); tree.add_node(11, 0); tree.add_node(12, 0); tree.add_node(13, 1);
+    tree.add_node(14, 1); tree.add_node(15, 2); tree.add_node(16, 4);
+    const std::vector<int> accepted = tree.find_accepted_nodes({10, 11, 14, 16});
+    REQUIRE((accepted == std::vector<int>{0, 1, 4, 6}));
+    std::vector<Tensor> kt, vt;
+    std::vector<std::vector<uint16_t>> kh, vh, want_k, want_v;
+    for (int l = 0; l < 2; ++l) {
+        kh.push_back(to_half(randn(size_t(hkv) * n_nodes * D, 8100 + l)));
+        vh.push_back(to_half(randn(size_t(hkv) * n_nodes * D, 8200 + l)));
+        kt.push_back(upload({hkv, n_nodes, D}, DataType::FP16, kh[l]));
+        vt.push_back(upload({hkv, n_nodes, D}, DataType::FP16, vh[l]));
+        want_k.push_back(download<uint16_t>(mgr.k_cache(l)));
+        want_v.push_back(download<uint16_t>(mgr.v_cache(l)));
+    }
+    const int free_before = mgr.num_free_blocks();
+    CHECK_OK(commit_tree_path(seq, original, accepted, kt, vt, backend()));
+    CHECK(seq.seq_len() == original + 4);                       // 33 tokens: 3 blocks
+    CHECK(seq.num_blocks() == 3 && mgr.num_free_blocks() >= free_before);
+    for (int l = 0; l < 2; ++l) {
+        for (int i = 0; i < 4; ++i) {
+            const int pos = original + i;
+            const size_t row = size_t(seq.block_table()[pos / bs]) * bs + pos % bs;
+            for (int h = 0; h < hkv; ++h)
+                for (int d = 0; d < D; ++d) {
+                    want_k[l][(row * hkv + h) * D + d] = kh[l][(size_t(h) * n_nodes + accepted[i]) * D + d];
+                    want_v[l][(row * hkv + h) * D + d] = vh[l][(size_t(h) * n_nodes + accepted[i]) * D + d];
+                }
+        }
+        CHECK(download<uint16_t>(mgr.k_cache(l)) == want_k[l]);   // bit exact, nothing else written
+        CHECK(download<uint16_t>(mgr.v_cache(l)) == want_v[l]);
+    }
+    const int outside[1] = {n_nodes};
+    CHECK_CODE(commit_tree_path(seq, original, outside, kt, vt, backend()), ErrorCode::InvalidArgument);
+    // an empty path only restores the length
+    CHECK_OK(commit_tree_path(seq, original, std::span<const int>(), kt, vt, backend()));
+    CHECK(seq.seq_len() == original);
+}
+
 int main(int argc, char** argv) {
     if (!backend()) {
         std::printf("no usable gfx950 GPU: skipping\n");

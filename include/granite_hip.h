@@ -163,6 +163,27 @@ int granite_hip_paged_kv_cache_append_ex(const void *new_k, const void *new_v, i
                                          uint32_t head_dim, uint32_t start_pos,
                                          uint32_t new_len, uint32_t block_size, int rounding);
 
+/* Commit of a speculation tree's accepted path.  After find_accepted_path
+ * (src/llm/speculation_tree.cpp:85-143) the runner only truncates the target
+ * cache to "original + accepted" (src/llm/speculative_runner.cpp:871-882),
+ * which assumes the tree's K/V had been appended in path order; the
+ * reference's attention_tree (transformer.mm:1870-2140, 2146-2402) appends
+ * nothing, so that step is unfinished upstream and this entry point defines
+ * it: row i of the cache range [start_pos, start_pos + num_accepted) receives
+ * tree node accepted_nodes[i] (device int32) of k_tree / v_tree, whose element
+ * (node s, head h, d) sits at s*src_tok_stride + h*src_head_stride + d
+ * ([num_kv_heads, num_nodes, D]: tok stride D, head stride num_nodes*D).  F16
+ * sources are copied bit for bit, F32 ones converted with `rounding`.  A node
+ * index outside [0, num_nodes) leaves its row unwritten.  block_table NULL:
+ * contiguous cache with row stride max_seq_len; else paged with block_size. */
+int granite_hip_kv_commit_accepted(const void *k_tree, const void *v_tree, int src_dtype,
+                                   int64_t src_tok_stride, int64_t src_head_stride,
+                                   uint32_t num_nodes, const int32_t *accepted_nodes,
+                                   uint32_t num_accepted, void *k_cache, void *v_cache,
+                                   const int32_t *block_table, uint32_t num_kv_heads,
+                                   uint32_t head_dim, uint32_t start_pos, uint32_t block_size,
+                                   uint32_t max_seq_len, int rounding);
+
 /* Gather of logical tokens [0, len) of one sequence out of the paged pools
  * into contiguous caches [num_kv_heads, max_seq_len, D] half (bit copy).  The
  * device form of the per-call gather in src/llm/transformer.mm:1750-1763 and

@@ -177,3 +177,61 @@ def test_null_and_bad_arguments(gpu):
     with pytest.raises(GraniteHipError) as e:
         gpu.paged_kv_cache_append(buf, buf, buf, buf, buf, 1, 128, 0, 1, 0)
     assert e.value.code == _capi.EINVAL
+
+
+@pytest.mark.parametrize("paged", [False, True])
+@pytest.mark.parametrize("src_dtype", [F16, F32])
+def test_kv_commit_accepted_path(gpu, oracle, paged, src_dtype):
+    """Commit of a speculation tree's accepted path: cache rows start_pos.. receive the accepted
+    nodes' K/V in path order.  The reference leaves this step unwritten (its runner only
+    truncates, src/llm/speculative_runner.cpp:871-882), so the semantics are this build's:
+    the expected cache is the oracle's append of the gathered rows."""
+    hkv, d, n_nodes, bs, start = 4, 128, 64, 16, 45
+    say(f"kv commit accepted paged={paged} src_dtype={src_dtype}")
+    rng = np.random.default_rng(91)
+    accepted = np.array([0, 3, 9, 10, 41, 63], np.int32)
+    tree_f32_k = (rng.standard_normal((hkv, n_nodes, d)) * 2).astype(np.float32)
+    tree_f32_v = (rng.standard_normal((hkv, n_nodes, d)) * 2).astype(np.float32)
+    if src_dtype == F16:
+        tk, tv = tree_f32_k.astype(np.float16).view(np.uint16), tree_f32_v.astype(np.float16).view(np.uint16)
+        rows_k, rows_v = tk[:, accepted], tv[:, accepted]                  # bit copy
+    else:
+        tk, tv = tree_f32_k, tree_f32_v
+        rows_k, rows_v = oracle.fp32_to_fp16(tk[:, accepted]), oracle.fp32_to_fp16(tv[:, accepted])
+    n = len(accepted)
+    if paged:
+        nblk = (start + n + bs - 1) // bs + 3
+        table = rng.permutation(nblk).astype(np.int32)
+        ck = np.full((nblk * bs, hkv, d), SENT, np.uint16)
+        cv = np.full((nblk * bs, hkv, d), SENT + 1, np.uint16)
+        want_k, want_v = ck.copy(), cv.copy()
+        for i in range(n):
+            pos = start + i
+            row = table[pos // bs] * bs + pos % bs
+            want_k[row], want_v[row] = rows_k[:, i], rows_v[:, i]
+        extra = dict(block_table=dev(table), block_size=bs)
+    else:
+        max_seq = 64
+        ck = np.full((hkv, max_seq, d), SENT, np.uint16)
+        cv = np.full((hkv, max_seq, d), SENT + 1, np.uint16)
+        want_k, want_v = ck.copy(), cv.copy()
+        want_k[:, start:start + n], want_v[:, start:start + n] = rows_k, rows_v
+        extra = dict(max_seq_len=max_seq)
+    dck, dcv, dtk, dtv, dacc = dev(ck), dev(cv), dev(tk), dev(tv), dev(accepted)
+    gpu.kv_commit_accepted(dtk, dtv, src_dtype, d, n_nodes * d, n_nodes, dacc, n, dck, dcv, hkv, d, start, **extra)
+    gpu.sync()
+    assert np.array_equal(dck.read(np.uint16, ck.shape), want_k)
+    assert np.array_equal(dcv.read(np.uint16, cv.shape), want_v)
+    # a node index outside the tree leaves its row unwritten; an empty path does nothing
+    bad = dev(np.array([1, -1, 64, 2], np.int32))
+    dck2, dcv2 = dev(ck), dev(cv)
+    gpu.kv_commit_accepted(dtk, dtv, src_dtype, d, n_nodes * d, n_nodes, bad, 4, dck2, dcv2, hkv, d, start, **extra)
+    gpu.kv_commit_accepted(dtk, dtv, src_dtype, d, n_nodes * d, n_nodes, bad, 0, dck2, dcv2, hkv, d, start, **extra)
+    gpu.sync()
+    got = dck2.read(np.uint16, ck.shape)
+    changed = (got != ck).any(axis=-1)
+    assert int(changed.sum()) == 2 * hkv   # only the two valid nodes' rows, one per head
+    if not paged:
+        with pytest.raises(GraniteHipError) as e:
+            gpu.kv_commit_accepted(dtk, dtv, src_dtype, d, n_nodes * d, n_nodes, dacc, n, dck, dcv, hkv, d, 60, **extra)
+        assert e.value.code == _capi.EOVERFLOW
