@@ -10,9 +10,12 @@
 // (fp32 scores and softmax, no epsilon, key k visible iff k <= start_pos + q;
 // tree: cache keys visible, tree key j visible iff j is q or an ancestor).
 //
-// Structure.  One workgroup of 8 waves (two per SIMD) per (query tile of 256
-// rows, query head, key split); a wave owns 32 query rows, and a K/V tile
-// staged in LDS serves all 256.  Workgroup ids are remapped so that the
+// Structure.  One workgroup of 8 waves (two per SIMD) per (256 query rows,
+// query head, key split); a wave owns 32 query rows, and a K/V tile staged in
+// LDS serves all 256.  The 256 rows are two runs of 128: the halves of one
+// query tile or, under a causal mask, the k-th run from the end and the k-th
+// from the start, so that every workgroup of a head has the same amount of
+// work.  Workgroup ids are remapped so that the
 // workgroups that stream the same K/V range (same KV head, same split) land on
 // the same XCD and share its L2.  Keys are walked in tiles of 64, each handled
 // as two 32-key sub-tiles.  Per sub-tile every wave computes, with
@@ -42,8 +45,8 @@
 // Data movement.  K/V tiles go global -> registers -> LDS; a thread moves two
 // 16-byte pieces of one key row of K and of V (one row lookup per thread and
 // tile).  What is loaded in one iteration is stored two iterations later (two
-// register sets), between the two phases of an iteration; row lookups run one
-// tile further ahead.  K is needed a tile earlier than V, so LDS holds three K
+// register sets), between the two phases of an iteration; block-table lookups
+// are issued two iterations before the loads that use them.  K is needed a tile earlier than V, so LDS holds three K
 // tiles (being finished, next, being written) and three V tiles (previous,
 // current, being written), which leaves one barrier per tile.  Both are stored
 // row-major as they lie in memory.  K rows have a pitch of 136 halves.  V rows
