@@ -62,11 +62,12 @@
 // elements.
 //
 // Softmax rescaling is lazy: probabilities are taken relative to a per-row
-// reference maximum that is only moved (and O, l rescaled) when the row
-// maximum of a sub-tile exceeds it by more than 2^8 (the probabilities of the
-// sub-tile still waiting for its second product are rescaled with them).
-// Results are identical up to rounding, P stays inside half range, and the
-// accumulators are left alone in almost every tile.
+// reference maximum that is not tracked tile by tile at all.  Only when the
+// probabilities of a sub-tile sum to 2^14 or more (or to infinity, as in the
+// first sub-tile, whose reference is still minus infinity) is the reference
+// moved to the row maximum, O and l rescaled and the sub-tile redone.  Results
+// are identical up to rounding, P stays inside half range, and neither the row
+// maximum nor the accumulator rescale is paid for in almost every tile.
 //
 // Algorithmic work: 4 * D flops per visible (query, key) pair.
 #include <cstdlib>
@@ -90,7 +91,7 @@ constexpr size_t kLdsBytes =
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-constexpr float kRescaleSlack = 8.0f;  // log2 of how far a probability may exceed 1
+constexpr float kProbLimit = 16384.0f;  // a row's probabilities of a sub-tile may sum to this much
 
 enum : int { kRowsContiguous = 0, kRowsPagedPow2 = 1, kRowsPagedAny = 2 };
 
@@ -402,48 +403,32 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
         return true;
     };
-    // Given the lane's maximum over a sub-tile's scores: the row maximum and, when a row
-    // outgrows the reference maximum, the rescale of m_ref, l and O.
-    // `pending` are probabilities that were taken relative to the old reference and have not
-    // been multiplied into O yet (the pipeline below keeps one sub-tile of them).
-    auto finish_max = [&](float mraw, half8 (*pending)[2]) {
+    // The reference maximum is not tracked tile by tile: probabilities are taken relative to
+    // the current reference, and only when those of a sub-tile sum to kProbLimit or more
+    // (or to infinity: the first sub-tile, whose reference is still minus infinity) is the
+    // reference moved to the row maximum and the sub-tile redone.  That keeps the maximum
+    // (16 comparisons, an exchange between the half waves) out of almost every sub-tile.
+    // A probability below kProbLimit is far inside half range; results are the same up to
+    // rounding because O, l and P always share one reference.
+    // rebase(): moves the reference up to cover the scores `sacc` and rescales l and O.
+    auto rebase = [&](const float16v& sacc) {
+        float mraw = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
         const LanePair both = half_wave_pair(mraw);
         const float m_tile = fmaxf(both.lo, both.hi) * p.scale_log2;
-        if (__any(m_tile > m_ref + kRescaleSlack)) {
-            const float m_new = fmaxf(m_ref, m_tile);
-            const float alpha = fast_exp2(m_ref - m_new);
-            m_ref = m_new;
-            l_run *= alpha;
-            if (pending) {
-                const _Float16 ah = static_cast<_Float16>(alpha);
+        const float m_new = fmaxf(m_ref, m_tile);
+        const float alpha = fast_exp2(m_ref - m_new);
+        m_ref = m_new;
+        l_run *= alpha;
 #pragma unroll
-                for (int u = 0; u < 2; u++)
+        for (int t = 0; t < 4; t++)
 #pragma unroll
-                    for (int j = 0; j < 8; j++) (*pending)[u][j] *= ah;
-            }
-#pragma unroll
-            for (int t = 0; t < 4; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
-        }
-    };
-    auto mask_and_max = [&](const TileInfo& ti, int sub, float16v& sacc) {
-        apply_mask(ti, sub, sacc);
-        float mraw = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
-        finish_max(mraw, nullptr);
-    };
-    auto mask_and_max_pending = [&](const TileInfo& ti, int sub, float16v& sacc, half8 (&pending)[2]) {
-        apply_mask(ti, sub, sacc);
-        float mraw = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
-        finish_max(mraw, &pending);
+            for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
     };
     // P^T = exp2(S^T * scale - m_ref) of a sub-tile as B operands of the second product;
     // adds to l.
-    auto probabilities = [&](const float16v& sacc, half8 (&bp)[2]) {
+    auto probabilities_once = [&](const float16v& sacc, half8 (&bp)[2]) -> float {
         float psum = 0.0f;
 #pragma unroll
         for (int u = 0; u < 2; u++) {
@@ -459,6 +444,14 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             w.z = pack_f16x2(pe[4], pe[5]);
             w.w = pack_f16x2(pe[6], pe[7]);
             bp[u] = as_half8(w);
+        }
+        return psum;
+    };
+    auto probabilities = [&](const float16v& sacc, half8 (&bp)[2]) {
+        float psum = probabilities_once(sacc, bp);
+        if (__any(!(psum < kProbLimit))) {
+            rebase(sacc);
+            psum = probabilities_once(sacc, bp);
         }
         l_run += psum;
     };
@@ -520,7 +513,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(i);
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        float psum = 0.0f, mraw = -INFINITY;
+        float psum = 0.0f;
         float pe[16];
         uint32_t pw[8];
         float tn = __builtin_fmaf(s_in[0], p.scale_log2, -m_ref);
@@ -544,23 +537,25 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = v_operand(i);
-        apply_mask(ti_q, sub_q, c);  // rare; the maximum of the new scores rides along below
+        apply_mask(ti_q, sub_q, c);  // rare
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             if (i + kRing - 1 < 8) ring[(i + kRing - 1) % kRing] = v_operand(i + kRing - 1);
             oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % kRing]),
                                                                  p_prev[i >> 2], oacc[i & 3], 0, 0, 0);
             softmax_step(8 + i);
-            mraw = fmaxf(fmaxf(mraw, c[2 * i]), c[2 * i + 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
         psum += pe[15];
         pw[7] = pack_f16x2(pe[14], pe[15]);
-        l_run += psum;
         p_out[0] = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
         p_out[1] = as_half8(uint4v{pw[4], pw[5], pw[6], pw[7]});
+        if (__any(!(psum < kProbLimit))) {  // rare: the reference has to move, redo the sub-tile
+            rebase(s_in);
+            psum = probabilities_once(s_in, p_out);
+        }
+        l_run += psum;
         s_out = c;
-        finish_max(mraw, &p_out);
     };
 
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
@@ -610,7 +605,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const TileInfo first = tile_info(t_begin);
         if (first.active) {
             scores(0, 0, s0);
-            mask_and_max(first, 0, s0);
+            apply_mask(first, 0, s0);
         }
     }
     uint32_t kb_cur = 0, kb_next = 1, kb_store = 2;  // K buffers of tiles it, it + 1, it + 2
@@ -643,13 +638,13 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             if (cur.active) {
                 scores(kb_cur, 1, s1);
                 probabilities(s0, p_new);
-                mask_and_max_pending(cur, 1, s1, p_new);
+                apply_mask(cur, 1, s1);
                 accumulate(vb_cur, 0, p_new);
                 probabilities(s1, p_old);
             }
             if (nxt.active) {
                 scores(kb_next, 0, s0);
-                mask_and_max_pending(nxt, 0, s0, p_old);
+                apply_mask(nxt, 0, s0);
             }
         }
         prev_active = cur.active;
