@@ -109,6 +109,42 @@ def test_chunked_prefill_over_paged_cache_small(gpu, oracle, prefix, chunk, bs, 
     assert_lse(lse.read(np.float32, (hq, chunk)), want_lse[0], "lse")
 
 
+@pytest.mark.parametrize("trial", range(12))
+def test_chunked_prefill_random_shapes(gpu, oracle, trial):
+    """Seeded random chunk lengths around the 128- and 256-row edges, prefixes, head counts and
+    block sizes, fp16 and fp32 queries: exercises the pairing of row runs, the key splits and
+    the first-tile handling of the softmax reference."""
+    rng = np.random.default_rng(500 + trial)
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    hq = hkv * int(rng.choice([1, 2, 4, 8]))
+    chunk = int(rng.choice([1, 31, 64, 127, 128, 129, 255, 256, 257, 384, 385, 511, 640]))
+    prefix = int(rng.choice([0, 1, 63, 64, 100, 500, 1200]))
+    bs = int(rng.choice([16, 32, 8, 12]))
+    say(f"chunked prefill random trial={trial} hq={hq} hkv={hkv} chunk={chunk} prefix={prefix} bs={bs}")
+    case = W.make_chunked_prefill(seed=trial, prefix_len=prefix, chunk=chunk, num_heads=hq, num_kv_heads=hkv,
+                                  block_size=bs, pool_slack=1.3, value_scale=1.0)
+    total = prefix + chunk
+    dk, dv, dt = dev(case.k_pool), dev(case.v_pool), dev(case.block_table)
+    gpu.paged_kv_cache_append_ex(dev(case.k_new), dev(case.v_new), F16, hkv * 128, 128, dk, dv, dt, hkv, 128,
+                                 prefix, chunk, bs)
+    gpu.sync()
+    pool_k, pool_v = dk.read(np.uint16, case.k_pool.shape), dv.read(np.uint16, case.v_pool.shape)
+    want, want_lse = oracle.attention_paged(case.q[None].astype(np.float32), pool_k, pool_v, case.block_table, bs,
+                                            total, prefix, case.scale)
+    f32 = trial % 3 == 0
+    q_host = case.q.astype(np.float32) if f32 else case.q
+    out = dev(np.zeros((chunk, hq, 128), np.float32 if f32 else np.float16))
+    lse = dev(np.zeros((hq, chunk), np.float32))
+    gpu.attention(q=dev(q_host), q_dtype=F32 if f32 else F16, q_tok_stride=hq * 128, q_head_stride=128, out=out,
+                  out_dtype=F32 if f32 else F16, out_tok_stride=hq * 128, out_head_stride=128, lse=lse, seq_q=chunk,
+                  num_heads=hq, num_kv_heads=hkv, head_dim=128, scale=case.scale, k_cache=dk, v_cache=dv,
+                  cache_len=total, block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
+    gpu.sync()
+    got = out.read(np.float32 if f32 else np.float16, (chunk, hq, 128)).astype(np.float32)
+    assert_close(got, want[0], "out", abs_tol=3e-3)
+    assert_lse(lse.read(np.float32, (hq, chunk)), want_lse[0], "lse")
+
+
 def test_chunked_prefill_config(gpu, oracle):
     """32768-token paged prefix (block 32), 512-token chunk, 64 q heads, 8 KV
     heads, values 0.5*N(0,1); append bit-exact, attention on sampled rows."""

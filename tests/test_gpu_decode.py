@@ -95,6 +95,38 @@ def test_batched_paged_decode_head_shapes(gpu, oracle, hq, hkv):
     assert np.all(got[~live] == -7.0)
 
 
+@pytest.mark.parametrize("trial", range(12))
+def test_batched_paged_decode_random_shapes(gpu, oracle, trial):
+    """Seeded random batches: head counts, group sizes, block sizes and length mixes (empty,
+    single-token, tile edges, long) that move the workers' range boundaries around."""
+    rng = np.random.default_rng(1000 + trial)
+    hkv = int(rng.choice([8, 16, 4, 2, 1, 3]))
+    hq = hkv * int(rng.choice([1, 2, 4, 8, 20]))
+    B = int(rng.integers(1, 24))
+    kind = trial % 4
+    if kind == 0:
+        lens = rng.integers(0, 200, B)
+    elif kind == 1:
+        lens = rng.integers(1, 2500, B)
+    elif kind == 2:
+        lens = np.where(rng.random(B) < 0.3, 0, rng.integers(1, 900, B))
+    else:
+        lens = rng.choice([1, 31, 32, 33, 63, 64, 65, 1024], B)
+    lens = lens.astype(np.int32)
+    lens[0] = max(lens[0], 3)
+    bs = int(rng.choice([16, 32, 8, 12]))
+    case = W.make_paged_decode(seed=trial, num_heads=hq, num_kv_heads=hkv, block_size=bs,
+                               ctx_max=int(max(lens.max(), 64)), seq_lens=lens)
+    say(f"batched paged decode random trial={trial} hq={hq} hkv={hkv} B={B} bs={bs} tokens={int(lens.sum())}")
+    want, want_lse = oracle.batched_paged_decode(case.q.astype(np.float32), case.k_pool, case.v_pool,
+                                                 case.block_tables, case.seq_lens, bs, case.scale)
+    got, got_lse = _run_batched(gpu, case, F16 if trial % 3 else F32)
+    live = lens > 0
+    assert_close(got[live], want[live], "out")
+    assert_lse(got_lse[live], want_lse[live], "lse")
+    assert np.all(got[~live] == -7.0)
+
+
 @pytest.mark.parametrize("chunk", [32, 128, 512, 1024])
 def test_batched_paged_decode_chunk_sizes_agree(gpu, oracle, chunk):
     lens = np.array([900, 31, 1500, 1024], np.int32)
