@@ -91,6 +91,7 @@ constexpr size_t kLdsBytes =
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+constexpr uint32_t kMaxFusedNodes = 256;  // largest tree whose ancestor mask a workgroup builds itself
 constexpr float kProbLimit = 16384.0f;  // a row's probabilities of a sub-tile may sum to this much
 
 enum : int { kRowsContiguous = 0, kRowsPagedPow2 = 1, kRowsPagedAny = 2 };
@@ -110,7 +111,8 @@ struct AttnParams {
     const uint16_t* k_extra;
     const uint16_t* v_extra;
     uint32_t extra_len;
-    const uint32_t* tree_mask;
+    const uint32_t* tree_mask;      // ancestor bit matrix in memory (trees beyond kMaxFusedNodes)
+    const int32_t* tree_parents;    // or: parent pointers, the workgroup builds its own matrix in LDS
     uint32_t mask_words;
     int mask_mode;
     uint32_t start_pos, seq_q, num_heads, group;
@@ -266,8 +268,31 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         }
     }
 
-    const uint32_t* mask_row =
-        p.tree_mask ? p.tree_mask + size_t(min(q_row, p.extra_len - 1)) * p.mask_words : nullptr;
+    // ---- tree mask.  Row i of the ancestor matrix has bit j set iff tree node i may attend
+    // node j: itself and its ancestors (src/llm/transformer.mm:822-840).  For trees of up to
+    // kMaxFusedNodes nodes every workgroup builds the matrix in LDS from the parent pointers:
+    // one thread per node walks the pointers (copied to LDS first), at most num_nodes steps,
+    // so a malformed array cannot hang it.  That saves a launch and keeps the mask reads out
+    // of the vector-memory queue.
+    __shared__ int32_t s_parent[kMaxFusedNodes];
+    __shared__ uint32_t s_rowmask[kMaxFusedNodes * (kMaxFusedNodes / 32)];
+    if (p.tree_parents) {  // uniform
+        for (uint32_t i = tid; i < p.extra_len; i += kThreads) s_parent[i] = p.tree_parents[i];
+        for (uint32_t i = tid; i < p.extra_len * p.mask_words; i += kThreads) s_rowmask[i] = 0;
+        __syncthreads();
+        if (tid < p.extra_len) {
+            uint32_t* row = s_rowmask + tid * p.mask_words;
+            row[tid >> 5] |= 1u << (tid & 31);
+            int32_t cur = s_parent[tid];
+            for (uint32_t step = 0; step < p.extra_len && cur >= 0 && cur < int32_t(p.extra_len); step++) {
+                row[uint32_t(cur) >> 5] |= 1u << (uint32_t(cur) & 31);
+                cur = s_parent[cur];
+            }
+        }
+        __syncthreads();
+    }
+    const uint32_t mask_row_index = min(q_row, p.extra_len - 1) * p.mask_words;
+    const uint32_t* mask_row = p.tree_mask ? p.tree_mask + mask_row_index : nullptr;
 
     float m_ref = kNegBig;  // reference maximum (log2 domain) the probabilities are relative to
     float l_run = 0.0f;     // lane-partial sum (the two k-groups are added at the end)
@@ -387,7 +412,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         uint32_t mw = 0xFFFFFFFFu;
         if (tree) {
             const uint32_t w = key0 >> 5;
-            mw = w < p.mask_words ? mask_row[w] : 0u;
+            mw = w >= p.mask_words ? 0u : (p.tree_parents ? s_rowmask[mask_row_index + w] : mask_row[w]);
         }
         const uint32_t limit = diagonal ? min(ti.seg_len, p.start_pos + q_row + 1) : ti.seg_len;
         // Element r is key 8 (r >> 2) + (r & 3) + 4 g of the sub-tile: everything that
@@ -902,7 +927,8 @@ int launch_attention(const granite_hip_attention_args& a) {
     }
     // One scratch request for everything (growing the scratch buffer moves it): the
     // tree mask first, the split-K partials behind it.
-    const bool tree = a.mask_mode == GRANITE_HIP_MASK_TREE;
+    const bool tree = a.mask_mode == GRANITE_HIP_MASK_TREE && a.extra_len > kMaxFusedNodes;
+    if (a.mask_mode == GRANITE_HIP_MASK_TREE && !tree) p.tree_parents = a.parents;
     const size_t mask_bytes =
         tree ? (size_t(a.extra_len) * p.mask_words * sizeof(uint32_t) + 255) & ~size_t(255) : 0;
     const size_t rows_total = n_splits > 1 ? size_t(n_splits) * a.num_heads * a.seq_q : 0;

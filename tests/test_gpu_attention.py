@@ -210,7 +210,10 @@ def _tree_gpu(gpu, case):
 
 
 @pytest.mark.parametrize("prefix,n,hq,hkv,bs", [(0, 1, 4, 4, 16), (0, 13, 8, 2, 16), (37, 5, 8, 2, 4),
-                                                (500, 64, 32, 8, 16), (64, 100, 4, 1, 16), (200, 130, 8, 2, 8)])
+                                                (500, 64, 32, 8, 16), (64, 100, 4, 1, 16), (200, 130, 8, 2, 8),
+                                                # 256 nodes: the largest tree whose mask the attention kernel
+                                                # builds itself; 257 and 300: through the mask kernel
+                                                (30, 256, 4, 2, 16), (30, 257, 4, 2, 16), (0, 300, 2, 1, 16)])
 def test_tree_attention_small(gpu, oracle, prefix, n, hq, hkv, bs):
     say(f"tree prefix={prefix} nodes={n} hq={hq} hkv={hkv} bs={bs}")
     case = W.make_tree(seed=prefix * 5 + n, prefix_len=prefix, num_nodes=n, num_heads=hq, num_kv_heads=hkv,
