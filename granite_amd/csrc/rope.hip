@@ -14,7 +14,7 @@
 // Layout as the reference kernel indexes it: Q [seq, Hq, D], K and V [seq, Hkv, D] float;
 // element pairs (2i, 2i+1) are rotated by angle (start_pos + s) * base^(-2i/D).
 //
-// A thread owns 4 consecutive floats (two pairs) of a token row and walks a run of 8 heads:
+// A thread owns 4 consecutive floats (two pairs) of a token row and walks a run of 4 heads:
 // one cos/sin lookup (or evaluation) serves them all, and the 32 threads of a row move 512
 // contiguous bytes per head.  The rotation is written with separately rounded
 // products and sums (no fused multiply-add), which is what the reference's CPU loop does,
@@ -58,7 +58,7 @@ __device__ __forceinline__ float2v rotate(float x0, float x1, float c, float s) 
     return r;
 }
 
-constexpr uint32_t kHeadsPerBlock = 8;
+constexpr uint32_t kHeadsPerBlock = 4;
 
 template <bool kNearest>
 __device__ __forceinline__ uint32_t half2_of(float a, float b) {
