@@ -329,21 +329,24 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         return row_finish<kRows>(p, r, min(it, n_tiles - 1) >= tiles_a);
     };
     // K and V of a tile are moved separately: K runs one tile ahead of V (see the loop).
-    auto load_k = [&](uint32_t it, uint32_t row, uint4v (&kreg)[2]) {
+    // load_k returns the element offset of its row; the V load of the same tile, issued one
+    // iteration later, starts from that offset instead of multiplying again.
+    auto load_k = [&](uint32_t it, uint32_t row, uint4v (&kreg)[2]) -> int64_t {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
         const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
-        const uint4v* src = reinterpret_cast<const uint4v*>(kb + int64_t(row) * stride);
+        const int64_t off = int64_t(row) * stride;
+        const uint4v* src = reinterpret_cast<const uint4v*>(kb + off);
         kreg[0] = src[0];
         kreg[1] = src[8];
+        return off;
     };
-    auto load_v = [&](uint32_t it, uint32_t row, uint4v (&vreg)[2]) {
+    auto load_v = [&](uint32_t it, int64_t off, uint4v (&vreg)[2]) {
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
-        const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
-        const uint4v* src = reinterpret_cast<const uint4v*>(vb + int64_t(row) * stride);
+        const uint4v* src = reinterpret_cast<const uint4v*>(vb + off);
         vreg[0] = src[0];
         vreg[1] = src[8];
     };
@@ -590,10 +593,10 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     const uint32_t r0 = tile_row(t_begin, tile_lookup(t_begin));
     const uint32_t r1 = tile_row(t_begin + 1, tile_lookup(t_begin + 1));
     const uint32_t r2 = tile_row(t_begin + 2, tile_lookup(t_begin + 2));
-    uint32_t row_v = tile_row(t_begin + 3, tile_lookup(t_begin + 3));  // of the tile whose V is loaded next
-    load_k(t_begin, r0, kreg_a);
-    load_v(t_begin, r0, vreg_a);
-    load_k(t_begin + 1, r1, kreg_b);
+    const uint32_t r3 = tile_row(t_begin + 3, tile_lookup(t_begin + 3));
+    const int64_t o0 = load_k(t_begin, r0, kreg_a);
+    load_v(t_begin, o0, vreg_a);
+    const int64_t o1 = load_k(t_begin + 1, r1, kreg_b);
     store_k(0, kreg_a);
     store_v(0, vreg_a);
     store_k(1, kreg_b);
@@ -606,13 +609,13 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     // pass are those of every other pass.
     // set a: K of tile t_begin + 2, V of t_begin + 1; set b: K of t_begin + 3, V of t_begin + 2
     __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move the lookups to the front)
-    load_k(t_begin + 2, r2, kreg_a);
-    load_v(t_begin + 1, r1, vreg_a);
+    const int64_t o2 = load_k(t_begin + 2, r2, kreg_a);
+    load_v(t_begin + 1, o1, vreg_a);
     __builtin_amdgcn_sched_barrier(0);
     RowLookup look_a = tile_lookup(t_begin + 4);
     __builtin_amdgcn_sched_barrier(0);
-    load_k(t_begin + 3, row_v, kreg_b);
-    load_v(t_begin + 2, r2, vreg_b);
+    int64_t off_v = load_k(t_begin + 3, r3, kreg_b);  // of the tile whose V is loaded next
+    load_v(t_begin + 2, o2, vreg_b);
     __builtin_amdgcn_sched_barrier(0);
     RowLookup look_b = tile_lookup(t_begin + 5);
     __builtin_amdgcn_sched_barrier(0);
@@ -651,9 +654,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         store_k(kb_store, kreg);  // K of tile it + 2
         store_v(vb_store, vreg);  // V of tile it + 1
         const uint32_t row_k = tile_row(it + 4, look);
-        load_k(it + 4, row_k, kreg);
-        load_v(it + 3, row_v, vreg);
-        row_v = row_k;
+        const int64_t off_k = load_k(it + 4, row_k, kreg);
+        load_v(it + 3, off_v, vreg);
+        off_v = off_k;
         look = tile_lookup(it + 6);
         if (fused) {
             fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new);
