@@ -48,8 +48,8 @@ CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
 # WRITE_SIZE unit); the summaries are under profiles/.
 MEASURED_TRAFFIC = {
     "paged_decode": 1146033048,    # decode_stream_kernel; algorithmic 1132236296
-    "prefill": 42584361,           # attention_tiles_kernel; algorithmic 41943040
-    "chunked_prefill": 179334980,  # attention_tiles_kernel; algorithmic 153092096
+    "prefill": 42595656,           # attention_tiles_kernel; algorithmic 41943040
+    "chunked_prefill": 179343219,  # attention_tiles_kernel; algorithmic 153092096
 }
 
 
@@ -386,6 +386,36 @@ def bench_copy_calibration(gpu, steps, warmup, cpu):
             "parity": {"bit_exact": bool(np.array_equal(got, np.transpose(pool, (1, 0, 2))))}}
 
 
+def bench_mfma_calibration(gpu, steps, warmup, cpu):
+    """The rate the matrix cores reach with nothing else running, on register operands: zeros
+    (the part keeps its peak clock) against normally distributed fp16 values (the power limit
+    holds the clock down), for both MFMA shapes.  The data-like rate is what an MFMA-bound
+    kernel can be compared with beside the published peak.  Not part of `--workload all`."""
+    from granite_amd import DeviceBuffer
+    rng = np.random.default_rng(11)
+    n = 1 << 20
+    data = {"zeros": np.zeros(n, np.float16),
+            "normal": (0.05 * rng.standard_normal(n, dtype=np.float32)).astype(np.float16)}
+    rates = {}
+    ms_total = 0.0
+    for kind, host in data.items():
+        buf = DeviceBuffer.from_numpy(host)
+        for shape in (32, 16):
+            flops = [0.0]
+
+            def step():
+                flops[0] = gpu.mfma_rate(buf, n, 20000, shape)
+
+            ms, _, _ = Timer(gpu).run(step, warmup, steps)
+            ms_total += ms
+            rates[f"{kind}_{shape}"] = round(flops[0] / (ms * 1e-3) / 1e12, 1)
+    return {"workload": "mfma_calibration_register_operands_8waves_per_cu", "metric": "mfma_TFLOPs",
+            "unit": "TFLOP/s", "value": rates["normal_32"], "ms_per_step": round(ms_total, 4),
+            "rates_TFLOPs": {"zeros_32x32x16": rates["zeros_32"], "zeros_16x16x32": rates["zeros_16"],
+                             "normal_32x32x16": rates["normal_32"], "normal_16x16x32": rates["normal_16"]},
+            "peak_TFLOPs": 2500.0}
+
+
 def bench_rope_append(gpu, steps, warmup, cpu):
     """The step in front of the attention path: rotate Q and K (the reference's cos/sin tables
     as input) and append the rotated K and V to the paged cache in the same pass.  Shape: a
@@ -474,7 +504,7 @@ WORKLOADS = {
     "decode_contiguous": bench_decode_contiguous,
     "rope_append": bench_rope_append,
 }
-EXTRA_WORKLOADS = {"copy_calibration": bench_copy_calibration}
+EXTRA_WORKLOADS = {"copy_calibration": bench_copy_calibration, "mfma_calibration": bench_mfma_calibration}
 
 
 def main() -> int:

@@ -445,6 +445,14 @@ int granite_hip_paged_kv_gather(void* dst_k, void* dst_v, const void* k_cache,
                                         head_dim, len, block_size, max_seq_len);
 }
 
+// ---- measurement aid ----------------------------------------------------------
+
+int granite_hip_mfma_rate(const void* operands_f16, uint64_t n_halves, uint32_t iterations,
+                          int shape, double* flops) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_mfma_rate(operands_f16, n_halves, iterations, shape, flops);
+}
+
 // ---- attention ------------------------------------------------------------
 
 int granite_hip_decode_attention(const granite_hip_decode_args* args) {

@@ -79,6 +79,8 @@ int launch_decode(const granite_hip_decode_args& a);
 int launch_attention(const granite_hip_attention_args& a);
 int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes);
 int launch_rope_append(const granite_hip_rope_args& a);
+int launch_mfma_rate(const void* operands, uint64_t n_halves, uint32_t iterations, int shape,
+                     double* flops);
 
 // ---- device helpers ------------------------------------------------------
 #if defined(__HIPCC__)

@@ -115,7 +115,8 @@ int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
  * reset_kernel_timing, get_kernel_timing_stats; include/granite/metal_compute.h:51-59).
  * While enabled every launch is bracketed by two events on the launch stream.
  * Names: "kv_append", "kv_gather", "decode_stream" or "decode_splitk",
- * "decode_merge", "attention_tiles", "attention_merge", "tree_mask", "rope_append".  granite_hip_kernel_timing_names() writes the
+ * "decode_merge", "attention_tiles", "attention_merge", "tree_mask", "rope_append",
+ * "mfma_rate".  granite_hip_kernel_timing_names() writes the
  * names seen so far, comma separated. */
 int granite_hip_enable_kernel_timing(int enable);
 int granite_hip_reset_kernel_timing(void);
@@ -380,6 +381,18 @@ typedef struct granite_hip_rope_args {
 } granite_hip_rope_args;
 
 int granite_hip_rope_append(const granite_hip_rope_args *args);
+
+/* Measurement aid with no counterpart in the reference: the rate the matrix cores
+ * reach when nothing else runs.  Two workgroups of eight waves per compute unit issue
+ * `iterations` passes of 16 v_mfma_f32_32x32x16_f16 (shape 32) or 32
+ * v_mfma_f32_16x16x32_f16 (shape 16) on register operands read once from
+ * operands_f16 (n_halves halves, a multiple of 8; lane i takes halves [16 i, 16 i + 16)
+ * modulo the buffer).  *flops receives the flops of the launch; time it with the events
+ * above or the kernel timer (name "mfma_rate").  With zeros the part keeps its peak clock;
+ * with data-like operands its power limit holds it lower, and that rate is the one an
+ * MFMA-bound kernel can be compared with. */
+int granite_hip_mfma_rate(const void *operands_f16, uint64_t n_halves, uint32_t iterations,
+                          int shape, double *flops);
 
 /* Bytes of device scratch the library keeps for split-K partial results. */
 size_t granite_hip_workspace_bytes(void);

@@ -235,3 +235,19 @@ def test_kv_commit_accepted_path(gpu, oracle, paged, src_dtype):
         with pytest.raises(GraniteHipError) as e:
             gpu.kv_commit_accepted(dtk, dtv, src_dtype, d, n_nodes * d, n_nodes, dacc, n, dck, dcv, hkv, d, 60, **extra)
         assert e.value.code == _capi.EOVERFLOW
+
+
+def test_mfma_rate_runs_and_checks_arguments(gpu):
+    """The matrix-core rate kernel (a measurement aid): finishes, reports its flops, and
+    refuses what its launch does not cover."""
+    say("mfma_rate")
+    n = 4096
+    buf = dev(np.ones(n, np.float16))
+    units = gpu.device_info().compute_units
+    for shape in (32, 16):
+        flops = gpu.mfma_rate(buf, n, 10, shape)
+        gpu.sync()
+        assert flops == 2 * units * 8 * 10 * 16 * 2 * 32 * 32 * 16
+    for n_halves, iterations, shape in ((12, 10, 32), (n, 0, 32), (n, 10, 8)):
+        with pytest.raises(GraniteHipError):
+            gpu.mfma_rate(buf, n_halves, iterations, shape)
