@@ -42,7 +42,8 @@
 // MFMAs costs next to nothing while the same work after a burst of MFMAs costs
 // its full time.
 //
-// Data movement.  K/V tiles go global -> registers -> LDS; a thread moves two
+// Data movement.  K/V tiles go global -> registers -> LDS (issued piecewise in the shadow
+// of the first phase's MFMAs); a thread moves two
 // 16-byte pieces of one key row of K and of V (one row lookup per thread and
 // tile).  What is loaded in one iteration is stored two iterations later (two
 // register sets), between the two phases of an iteration; block-table lookups
@@ -350,6 +351,14 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         vreg[0] = src[0];
         vreg[1] = src[8];
     };
+    auto store_k_piece = [&](uint32_t buf, const uint4v (&kreg)[2], int piece) {
+        uint4v* dst = reinterpret_cast<uint4v*>(s_k0 + buf * kKTileHalves + k_st);
+        dst[8 * piece] = kreg[piece];
+    };
+    auto store_v_piece = [&](uint32_t buf, const uint4v (&vreg)[2], int piece) {
+        uint16_t* sv = s_v0 + buf * kVTileHalves;
+        *reinterpret_cast<uint4v*>(sv + (piece ? v_st2 : v_st)) = vreg[piece];
+    };
     auto store_k = [&](uint32_t buf, const uint4v (&kreg)[2]) {
         uint4v* dst = reinterpret_cast<uint4v*>(s_k0 + buf * kKTileHalves + k_st);
         dst[0] = kreg[0];
@@ -516,11 +525,13 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
     // transcendentals run beside it, so a few vector instructions between MFMAs are free
     // while the same instructions after a burst of MFMAs are not.  The scheduling barriers
     // and the empty asm statements keep the compiler from regrouping or sinking the slices.
+    // side(step) is called after the vector work of every step (0..15) for work of the
+    // caller's that should issue in the shadow of the MFMAs (the tile staging).
     // Operands are fetched from LDS two steps ahead.  Step e scales element e + 1, takes the
     // exponential of element e and sums / packs element e - 1.
     auto fused_phase = [&](const TileInfo& ti_q, uint32_t kbuf, int sub_q, float16v& s_out,
                            const float16v& s_in, half8 (&p_out)[2], uint32_t vbuf, int sub_v,
-                           const half8 (&p_prev)[2]) {
+                           const half8 (&p_prev)[2], auto&& side) {
         const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
         const uint16_t* sv = s_v0 + vbuf * kVTileHalves + 32 * sub_v * kVPitch;
         auto k_operand = [&](int s8) -> uint4v {
@@ -561,6 +572,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             if constexpr (kQF32)
                 c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq_lo[s8], c, 0, 0, 0);
             softmax_step(s8);
+            side(s8);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -572,6 +584,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % kRing]),
                                                                  p_prev[i >> 2], oacc[i & 3], 0, 0, 0);
             softmax_step(8 + i);
+            side(8 + i);
             __builtin_amdgcn_sched_barrier(0);
         }
         psum += pe[15];
@@ -643,24 +656,31 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const TileInfo cur = tile_info(it);
         const TileInfo nxt = tile_info(it + 1);
         const bool fused = prev_active && cur.active && nxt.active;  // the common case
+        // Staging, on every path (indices clamp at the last tile; stores past the last tile go
+        // to buffers nobody reads any more): what is stored now was requested two iterations
+        // ago (the register set alternates), and the target buffers (K of tile it - 1, V of
+        // tile it - 2) have been free since the last barrier.  In a fused iteration its
+        // pieces are spread over the second half of the first phase, one per MFMA, so that
+        // the matrix cores do not idle while the waves of a SIMD store and load together.
+        auto staging = [&](int piece) {
+            if (piece == 0) store_k_piece(kb_store, kreg, 0);  // K of tile it + 2
+            if (piece == 1) store_k_piece(kb_store, kreg, 1);
+            if (piece == 2) store_v_piece(vb_store, vreg, 0);  // V of tile it + 1
+            if (piece == 3) store_v_piece(vb_store, vreg, 1);
+            if (piece == 4) {
+                const uint32_t row_k = tile_row(it + 4, look);
+                const int64_t off_k = load_k(it + 4, row_k, kreg);
+                load_v(it + 3, off_v, vreg);
+                off_v = off_k;
+            }
+            if (piece == 5) look = tile_lookup(it + 6);
+        };
         if (fused) {
-            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old);
-        }
-        // Staging, unconditional (indices clamp at the last tile): loads inside a branch would
-        // force a full wait at the join; stores past the last tile go to buffers nobody reads
-        // any more.  It sits between the two phases; what is stored now was requested two
-        // iterations ago (the register set alternates), and the target buffers (K of tile
-        // it - 1, V of tile it - 2) have been free since the last barrier.
-        store_k(kb_store, kreg);  // K of tile it + 2
-        store_v(vb_store, vreg);  // V of tile it + 1
-        const uint32_t row_k = tile_row(it + 4, look);
-        const int64_t off_k = load_k(it + 4, row_k, kreg);
-        load_v(it + 3, off_v, vreg);
-        off_v = off_k;
-        look = tile_lookup(it + 6);
-        if (fused) {
-            fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new);
+            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old, [&](int step) { staging(step - 8); });
+            fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new, [](int) {});
         } else {
+#pragma unroll
+            for (int piece = 0; piece < 6; piece++) staging(piece);
             // the same three stages one after the other, each only where it applies
             if (prev_active) accumulate(vb_prev, 1, p_old);
             if (cur.active) {
