@@ -46,7 +46,7 @@
 // of the first phase's MFMAs); a thread moves two
 // 16-byte pieces of one key row of K and of V (one row lookup per thread and
 // tile).  What is loaded in one iteration is stored two iterations later (two
-// register sets), between the two phases of an iteration; block-table lookups
+// register sets); block-table lookups
 // are issued two iterations before the loads that use them.  K is needed a tile earlier than V, so LDS holds three K
 // tiles (being finished, next, being written) and three V tiles (previous,
 // current, being written), which leaves one barrier per tile.  Both are stored
