@@ -48,8 +48,8 @@ CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
 # WRITE_SIZE unit); the summaries are under profiles/.
 MEASURED_TRAFFIC = {
     "paged_decode": 1146033048,    # decode_stream_kernel; algorithmic 1132236296
-    "prefill": 42595656,           # attention_tiles_kernel; algorithmic 41943040
-    "chunked_prefill": 179343219,  # attention_tiles_kernel; algorithmic 153092096
+    "prefill": 42603693,           # attention_tiles_kernel; algorithmic 41943040
+    "chunked_prefill": 179373956,  # attention_tiles_kernel; algorithmic 153092096
 }
 
 
