@@ -13,7 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libgranite_hip.so"
 
 # constants of granite_hip.h
 OK = 0
-EINVAL, ENOTINIT, ENOMEM, EUNSUPPORTED, ENULL, EOVERFLOW = -1, -2, -3, -4, -5, -6
+EINVAL, ENOTINIT, ENOMEM, EUNSUPPORTED, ENULL, EOVERFLOW, ESCRATCH = -1, -2, -3, -4, -5, -6, -7
 F32, F16 = 0, 1
 ROUND_TRUNCATE, ROUND_NEAREST = 0, 1
 MEM_DEVICE, MEM_SHARED, MEM_MANAGED = 0, 1, 2
@@ -175,6 +175,11 @@ SIGNATURES = {
     "granite_hip_rope_append": (_int, [C.POINTER(RopeArgs)]),
     "granite_hip_mfma_rate": (_int, [_vp, C.c_uint64, _u32, _int, C.POINTER(C.c_double)]),
     "granite_hip_workspace_bytes": (C.c_size_t, []),
+    "granite_hip_reserve_workspace": (_int, [C.c_size_t]),
+    "granite_hip_decode_workspace_required": (_int, [C.POINTER(DecodeArgs), C.POINTER(C.c_size_t)]),
+    "granite_hip_attention_workspace_required": (_int, [C.POINTER(AttentionArgs), C.POINTER(C.c_size_t)]),
+    "granite_hip_decode_attention_ws": (_int, [C.POINTER(DecodeArgs), _vp, C.c_size_t]),
+    "granite_hip_attention_ws": (_int, [C.POINTER(AttentionArgs), _vp, C.c_size_t]),
 }
 
 _lib = None

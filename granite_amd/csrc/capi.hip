@@ -21,8 +21,9 @@ Context& ctx() {
 int ensure_workspace(size_t bytes) {
     Context& c = ctx();
     if (bytes <= c.workspace_bytes) return GRANITE_HIP_OK;
-    // Earlier launches may still read the old buffer.
-    GHIP_CHECK(hipStreamSynchronize(c.stream));
+    // Earlier launches, on this stream or on one the caller used before
+    // granite_hip_set_stream, may still use the old buffer.
+    GHIP_CHECK(hipDeviceSynchronize());
     if (c.workspace) GHIP_CHECK(hipFree(c.workspace));
     c.workspace = nullptr;
     c.workspace_bytes = 0;
@@ -34,6 +35,24 @@ int ensure_workspace(size_t bytes) {
         return GRANITE_HIP_ENOMEM;
     }
     c.workspace_bytes = want;
+    return GRANITE_HIP_OK;
+}
+
+int take_scratch(const ScratchSource& src, size_t need, void** ws) {
+    *ws = nullptr;
+    if (src.query) {
+        *src.query = need;
+        return GRANITE_HIP_OK;
+    }
+    if (src.fixed) {
+        if (need > src.fixed_bytes) return GRANITE_HIP_ESCRATCH;
+        if (reinterpret_cast<uintptr_t>(src.fixed) & 255) return GRANITE_HIP_EINVAL;
+        *ws = src.fixed;
+        return GRANITE_HIP_OK;
+    }
+    int rc = ensure_workspace(need);
+    if (rc != GRANITE_HIP_OK) return rc;
+    *ws = ctx().workspace;
     return GRANITE_HIP_OK;
 }
 
@@ -116,6 +135,7 @@ const char* granite_hip_error_string(int code) {
         case GRANITE_HIP_EUNSUPPORTED: return "NotImplemented";
         case GRANITE_HIP_ENULL: return "NullPointer";
         case GRANITE_HIP_EOVERFLOW: return "InvalidArgument: KV cache overflow";
+        case GRANITE_HIP_ESCRATCH: return "InvalidArgument: the launch needs more scratch memory than the buffer given holds";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -253,7 +273,19 @@ int granite_hip_sync(void) {
 
 int granite_hip_set_stream(void* stream) {
     GHIP_REQUIRE_INIT();
-    ctx().stream = stream ? static_cast<hipStream_t>(stream) : ctx().own_stream;
+    ghip::Context& c = ctx();
+    hipStream_t next = stream ? static_cast<hipStream_t>(stream) : c.own_stream;
+    if (next == c.stream) return GRANITE_HIP_OK;
+    // All launches share one scratch buffer: whatever is still queued on the old stream
+    // has to finish before a launch on the new one may overwrite its partials.
+    ghip::resolve_timings();
+    hipEvent_t done = nullptr;
+    GHIP_CHECK(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+    hipError_t e = hipEventRecord(done, c.stream);
+    if (e == hipSuccess) e = hipStreamWaitEvent(next, done, 0);
+    (void)hipEventDestroy(done);  // released once the recorded work has completed
+    if (e != hipSuccess) return static_cast<int>(e);
+    c.stream = next;
     return GRANITE_HIP_OK;
 }
 
@@ -345,6 +377,49 @@ int granite_hip_rope_multihead(void* q, void* k, uint32_t num_heads_q, uint32_t 
 }
 
 size_t granite_hip_workspace_bytes(void) { return ctx().workspace_bytes; }
+
+int granite_hip_reserve_workspace(size_t bytes) {
+    GHIP_REQUIRE_INIT();
+    return ghip::ensure_workspace(bytes);
+}
+
+int granite_hip_decode_workspace_required(const granite_hip_decode_args* args, size_t* bytes) {
+    GHIP_REQUIRE_INIT();
+    if (!args || !bytes) return GRANITE_HIP_ENULL;
+    ghip::ScratchSource src;
+    src.query = bytes;
+    return ghip::launch_decode(*args, src);
+}
+
+int granite_hip_attention_workspace_required(const granite_hip_attention_args* args, size_t* bytes) {
+    GHIP_REQUIRE_INIT();
+    if (!args || !bytes) return GRANITE_HIP_ENULL;
+    ghip::ScratchSource src;
+    src.query = bytes;
+    return ghip::launch_attention(*args, src);
+}
+
+int granite_hip_decode_attention_ws(const granite_hip_decode_args* args, void* workspace,
+                                    size_t workspace_bytes) {
+    GHIP_REQUIRE_INIT();
+    if (!args) return GRANITE_HIP_ENULL;
+    if (!workspace) return ghip::launch_decode(*args);
+    ghip::ScratchSource src;
+    src.fixed = workspace;
+    src.fixed_bytes = workspace_bytes;
+    return ghip::launch_decode(*args, src);
+}
+
+int granite_hip_attention_ws(const granite_hip_attention_args* args, void* workspace,
+                             size_t workspace_bytes) {
+    GHIP_REQUIRE_INIT();
+    if (!args) return GRANITE_HIP_ENULL;
+    if (!workspace) return ghip::launch_attention(*args);
+    ghip::ScratchSource src;
+    src.fixed = workspace;
+    src.fixed_bytes = workspace_bytes;
+    return ghip::launch_attention(*args, src);
+}
 
 int granite_hip_enable_kernel_timing(int enable) {
     GHIP_REQUIRE_INIT();

@@ -25,9 +25,26 @@ struct Context {
 
 Context& ctx();
 
-// Grows the scratch buffer to at least `bytes` (stream-ordered with respect
-// to earlier launches: the old buffer is released only after a sync).
+// Grows the scratch buffer to at least `bytes`.  Growing waits for the whole
+// device first (launches on any stream may still use the old buffer), frees
+// and allocates; callers that must not stall reserve once up front
+// (granite_hip_reserve_workspace) or bring their own scratch.
 int ensure_workspace(size_t bytes);
+
+// Where a launch takes its scratch memory (split-K partials, plans, tree masks) from.
+//   default            the library workspace, grown when too small
+//   fixed != nullptr   that buffer and nothing else: no allocation, no synchronisation;
+//                      a launch that needs more fails with GRANITE_HIP_ESCRATCH
+//   query != nullptr   nothing is launched; *query receives the bytes the launch needs
+struct ScratchSource {
+    void* fixed = nullptr;
+    size_t fixed_bytes = 0;
+    size_t* query = nullptr;
+};
+
+// Resolves `need` bytes against `src`.  Returns GRANITE_HIP_OK with *ws set (nullptr for a
+// query, in which case the caller returns at once), or an error code.
+int take_scratch(const ScratchSource& src, size_t need, void** ws);
 
 #define GHIP_CHECK(expr)                               \
     do {                                               \
@@ -75,8 +92,8 @@ int launch_kv_append_paged(const void* new_k, const void* new_v, int src_dtype,
 int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const void* v_cache,
                            const int32_t* block_table, uint32_t num_kv_heads, uint32_t head_dim,
                            uint32_t len, uint32_t block_size, uint32_t max_seq_len);
-int launch_decode(const granite_hip_decode_args& a);
-int launch_attention(const granite_hip_attention_args& a);
+int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch = {});
+int launch_attention(const granite_hip_attention_args& a, const ScratchSource& scratch = {});
 int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes);
 int launch_rope_append(const granite_hip_rope_args& a);
 int launch_mfma_rate(const void* operands, uint64_t n_halves, uint32_t iterations, int shape,

@@ -304,12 +304,13 @@ static bool use_stream_kernel() {
     return value;
 }
 
-int launch_decode(const granite_hip_decode_args& a) {
+int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch) {
     if (!a.q || !a.k_cache || !a.v_cache || !a.out) return GRANITE_HIP_ENULL;
-    if (a.head_dim != kHeadDim) return GRANITE_HIP_EINVAL;
+    if (a.head_dim != kHeadDim) return GRANITE_HIP_EUNSUPPORTED;
     if (a.num_heads == 0 || a.num_kv_heads == 0 || a.num_heads % a.num_kv_heads != 0)
         return GRANITE_HIP_EINVAL;
     if (a.q_dtype != GRANITE_HIP_F32 && a.q_dtype != GRANITE_HIP_F16) return GRANITE_HIP_EINVAL;
+    if (scratch.query) *scratch.query = 0;
     if (a.batch_size == 0) return GRANITE_HIP_OK;
 
     DecodeParams p{};
@@ -367,20 +368,23 @@ int launch_decode(const granite_hip_decode_args& a) {
         const uint64_t units = uint64_t(p.batch) * ((p.max_tokens + kTile - 1) / kTile) *
                                p.num_kv_heads * p.q_groups;
         if (units < (1ull << 31) && decode_stream_supports(p.batch))
-            return launch_decode_stream(p, qf32, rows);
+            return launch_decode_stream(p, qf32, rows, scratch);
     }
 
+    if (p.max_chunks > 65535u * 32 || p.batch > 65535u) return GRANITE_HIP_EINVAL;
     int rc = GRANITE_HIP_OK;
     if (p.max_chunks > 1) {
         const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;
         const size_t need = slots * (kHeadDim + 2) * sizeof(float);
-        rc = ensure_workspace(need);
-        if (rc != GRANITE_HIP_OK) return rc;
-        p.part_o = static_cast<float*>(ctx().workspace);
+        void* ws = nullptr;
+        rc = take_scratch(scratch, need, &ws);
+        if (rc != GRANITE_HIP_OK || scratch.query) return rc;
+        p.part_o = static_cast<float*>(ws);
         p.part_ml = p.part_o + slots * kHeadDim;
+    } else if (scratch.query) {
+        return GRANITE_HIP_OK;  // one chunk per sequence: the kernel writes the result itself
     }
 
-    if (p.max_chunks > 65535u * 32 || p.batch > 65535u) return GRANITE_HIP_EINVAL;
     dim3 grid(p.max_chunks, p.num_kv_heads * p.q_groups, p.batch);
     dim3 block(kWavesPerWG * kWave);
     hipStream_t st = ctx().stream;

@@ -19,8 +19,8 @@ struct DecodeParams {
     const uint16_t* v;
     const int32_t* tables;
     const int32_t* seq_lens;
-    float* part_o;   // [B, Hq, max_chunks, D]
-    float* part_ml;  // [B, Hq, max_chunks, 2]
+    float* part_o;   // chunk kernel: [B, Hq, max_chunks, D]; stream kernel: [piece, part_cap, D]
+    float* part_ml;  // same, [.., 2] = (max, sum)
     float* out;
     float* lse;
     uint32_t batch, num_heads, num_kv_heads, group, q_groups;
@@ -29,7 +29,8 @@ struct DecodeParams {
     int64_t tok_stride, head_stride;
     uint32_t max_tokens;  // bound on any sequence length
     uint32_t chunk_tokens, max_chunks;
-    uint32_t workers, min_per;  // stream kernel: waves in the grid, smallest share of a wave
+    uint32_t workers, min_per;  // stream kernel: workers in the grid, smallest share of one
+    uint32_t part_cap;          // stream kernel: query heads a piece slot holds
     float scale_log2;
 };
 
@@ -73,6 +74,6 @@ constexpr uint32_t kPlanHeader = 4;  // words in front of prefix[]
 // (60 KiB at most); larger batches go through the chunk kernel.
 constexpr uint32_t kStreamMaxPrefix = 7680;
 bool decode_stream_supports(uint32_t batch);
-int launch_decode_stream(DecodeParams p, bool q_f32, int rows);
+int launch_decode_stream(DecodeParams p, bool q_f32, int rows, const ScratchSource& scratch);
 
 }  // namespace ghip

@@ -22,6 +22,14 @@
 // (m, l, O) for the part it covered; the merge kernel combines the partials of
 // a (sequence, head), whose positions follow from the same arithmetic.
 //
+// Partials are stored compactly.  Walking the flat list, a new piece (one worker's
+// part of one (sequence, list head) segment) begins at every worker boundary and at
+// every segment boundary, so the pieces are numbered without collision by
+// worker + segment, segment = sequence * lists + list head: from one piece to the
+// next the worker or the segment grows, and neither ever shrinks.  There are
+// therefore workers + batch * lists piece slots however long the sequences may
+// become, each holding the query heads of one list head.
+//
 // There is no separate planning launch: every workgroup scans the sequence
 // lengths into tile counts and their prefix sums itself, in LDS (a few hundred
 // nanoseconds for a batch of 64), and looks everything up there afterwards, so
@@ -77,6 +85,14 @@ __device__ __forceinline__ void advance(const DecodeParams& p, const uint32_t* l
 
 // Heads of one list entry in the rows shape: two per wave.
 constexpr uint32_t kPairHeads = 2 * kWavesPerWG;
+
+// First query head of list head `lh`: a list head is one virtual head
+// (kv_head * q_groups + q_group, up to 16 query heads) or, in the rows shape, 8
+// consecutive ones; the query heads of consecutive virtual heads are consecutive.
+__device__ __forceinline__ uint32_t list_first_head(const DecodeParams& p, uint32_t lh, bool pair) {
+    const uint32_t v0 = pair ? lh * kPairHeads : lh;
+    return (v0 / p.q_groups) * p.group + (v0 % p.q_groups) * 16;
+}
 
 struct TileRegs {
     half8 ka[2][4];
@@ -315,11 +331,11 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
         const uint32_t kvh = vh / p.q_groups, qg = vh % p.q_groups;
         const uint32_t q_in_group = qg * 16 + n;
         if (q_in_group < p.group) {
-            // slot = this worker's rank among the workers that touch (b, list head)
-            const uint32_t u_start = prefix_u(c.b) * lists + c.vh * c.nt;
-            const uint32_t slot = worker - u_start / per;
-            const size_t head = size_t(c.b) * p.num_heads + kvh * p.group + q_in_group;
-            const size_t at = head * p.max_chunks + slot;
+            // piece slot = worker + segment; inside it, the query head counted from the
+            // first one of the list head
+            const uint32_t piece = worker + c.b * lists + c.vh;
+            const uint32_t local = kvh * p.group + q_in_group - list_first_head(p, c.vh, kPair);
+            const size_t at = size_t(piece) * p.part_cap + local;
             float* po = p.part_o + at * kHeadDim + 32 * g;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -446,21 +462,27 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
     const uint32_t vheads = p.num_kv_heads * p.q_groups;
     const uint32_t kvh = qh / p.group, qg = (qh % p.group) / 16;
     const uint32_t heads_per_list = p.plan[2];  // 1 (flat list) or 8 (rows)
+    const uint32_t lists = vheads / heads_per_list;
     const uint32_t vh = (kvh * p.q_groups + qg) / heads_per_list;
-    const uint32_t u_start = prefix[b] * (vheads / heads_per_list) + vh * nt;
-    const uint32_t n_parts = (u_start + nt - 1) / per - u_start / per + 1;
+    const uint32_t u_start = prefix[b] * lists + vh * nt;
+    const uint32_t first_worker = u_start / per;
+    const uint32_t n_parts = (u_start + nt - 1) / per - first_worker + 1;
     const size_t head = size_t(b) * p.num_heads + qh;
-    const float* ml = p.part_ml + head * p.max_chunks * 2;
-    const float* po = p.part_o + head * p.max_chunks * kHeadDim;
+    // piece c of this segment sits in slot first_worker + c + segment (see the stream kernel)
+    const size_t at0 = size_t(first_worker + b * lists + vh) * p.part_cap +
+                       (qh - list_first_head(p, vh, heads_per_list > 1));
+    const float* ml = p.part_ml + at0 * 2;
+    const float* po = p.part_o + at0 * kHeadDim;
+    const size_t step = p.part_cap;  // slots of consecutive pieces are part_cap heads apart
     const uint32_t d = threadIdx.x;
 
     float mx = kNegBig;
-    for (uint32_t c = 0; c < n_parts; c++) mx = fmaxf(mx, ml[2 * c]);
+    for (uint32_t c = 0; c < n_parts; c++) mx = fmaxf(mx, ml[2 * c * step]);
     float o = 0.0f, l = 0.0f;
     for (uint32_t c = 0; c < n_parts; c++) {
-        const float f = fast_exp2(ml[2 * c] - mx);
-        l += ml[2 * c + 1] * f;
-        o += po[size_t(c) * kHeadDim + d] * f;
+        const float f = fast_exp2(ml[2 * c * step] - mx);
+        l += ml[2 * c * step + 1] * f;
+        o += po[c * step * kHeadDim + d] * f;
     }
     p.out[head * kHeadDim + d] = o / l;
     if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
@@ -470,27 +492,32 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
 
 bool decode_stream_supports(uint32_t batch) { return batch + 1 <= kStreamMaxPrefix; }
 
-int launch_decode_stream(DecodeParams p, bool q_f32, int rows) {
+int launch_decode_stream(DecodeParams p, bool q_f32, int rows, const ScratchSource& scratch) {
     if (!decode_stream_supports(p.batch)) return GRANITE_HIP_EINVAL;
     // One workgroup per CU, one wave per SIMD.  A worker is a workgroup when the heads come
     // in groups of 8 (the rows shape), else a wave.
     const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
     const uint32_t wgs = cus;
-    const bool pair = (p.num_kv_heads * p.q_groups) % kPairHeads == 0;
+    const uint32_t vheads = p.num_kv_heads * p.q_groups;
+    const bool pair = vheads % kPairHeads == 0;
     const uint32_t workers = pair ? wgs : wgs * kWavesPerWG;
-    // Smallest range a worker may get: it bounds the partial slots per (sequence, head) to
-    // about 32 however short the batch is, and is never above chunk_tokens.
+    // Smallest range a worker may get: it keeps a short batch from being cut into ranges
+    // of a tile or two, and is never above chunk_tokens.
     const uint32_t max_tiles = (p.max_tokens + kTile - 1) / kTile;
     const uint32_t min_per = min(max(p.chunk_tokens / kTile, 1u), max((max_tiles + 31) / 32, 1u));
-    p.max_chunks = (max_tiles + min_per - 1) / min_per + 2;  // partial slots per (sequence, head)
 
-    const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;
+    // Partial results: one slot per piece (worker + segment), each with room for the query
+    // heads of a list head.
+    const uint32_t lists = pair ? vheads / kPairHeads : vheads;
+    p.part_cap = (pair ? kPairHeads : 1u) * min(p.group, 16u);
+    const size_t slots = (size_t(workers) + size_t(p.batch) * lists) * p.part_cap;
     const size_t plan_words = kPlanHeader + size_t(p.batch) + 1;
     const size_t plan_bytes = (plan_words * sizeof(uint32_t) + 255) & ~size_t(255);
     const size_t need = plan_bytes + slots * (kHeadDim + 2) * sizeof(float);
-    int rc = ensure_workspace(need);
-    if (rc != GRANITE_HIP_OK) return rc;
-    char* ws = static_cast<char*>(ctx().workspace);
+    void* ws_ptr = nullptr;
+    int rc = take_scratch(scratch, need, &ws_ptr);
+    if (rc != GRANITE_HIP_OK || scratch.query) return rc;
+    char* ws = static_cast<char*>(ws_ptr);
     p.plan = reinterpret_cast<uint32_t*>(ws);
     p.part_o = reinterpret_cast<float*>(ws + plan_bytes);
     p.part_ml = p.part_o + slots * kHeadDim;

@@ -870,14 +870,15 @@ int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_
     return launch_status();
 }
 
-int launch_attention(const granite_hip_attention_args& a) {
+int launch_attention(const granite_hip_attention_args& a, const ScratchSource& scratch) {
     if (!a.q || !a.out) return GRANITE_HIP_ENULL;
-    if (a.head_dim != kHeadDim) return GRANITE_HIP_EINVAL;
+    if (a.head_dim != kHeadDim) return GRANITE_HIP_EUNSUPPORTED;
     if (a.num_heads == 0 || a.num_kv_heads == 0 || a.num_heads % a.num_kv_heads != 0)
         return GRANITE_HIP_EINVAL;
     if ((a.q_dtype != GRANITE_HIP_F32 && a.q_dtype != GRANITE_HIP_F16) ||
         (a.out_dtype != GRANITE_HIP_F32 && a.out_dtype != GRANITE_HIP_F16))
         return GRANITE_HIP_EINVAL;
+    if (scratch.query) *scratch.query = 0;
     if (a.seq_q == 0) return GRANITE_HIP_OK;
     if (a.cache_len + a.extra_len == 0) return GRANITE_HIP_EINVAL;
     if (a.cache_len > 0 && (!a.k_cache || !a.v_cache)) return GRANITE_HIP_ENULL;
@@ -956,10 +957,15 @@ int launch_attention(const granite_hip_attention_args& a) {
         tree ? (size_t(a.extra_len) * p.mask_words * sizeof(uint32_t) + 255) & ~size_t(255) : 0;
     const size_t rows_total = n_splits > 1 ? size_t(n_splits) * a.num_heads * a.seq_q : 0;
     const size_t need = mask_bytes + rows_total * (kHeadDim + 2) * sizeof(float);
+    if (scratch.query) {
+        *scratch.query = need;
+        return GRANITE_HIP_OK;
+    }
     if (need > 0) {
-        int rc = ensure_workspace(need);
+        void* ws_ptr = nullptr;
+        int rc = take_scratch(scratch, need, &ws_ptr);
         if (rc != GRANITE_HIP_OK) return rc;
-        char* ws = static_cast<char*>(ctx().workspace);
+        char* ws = static_cast<char*>(ws_ptr);
         if (tree) {
             uint32_t* mask = reinterpret_cast<uint32_t*>(ws);
             rc = launch_tree_mask(a.parents, mask, a.extra_len);

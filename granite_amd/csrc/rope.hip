@@ -202,6 +202,11 @@ int launch_rope_append(const granite_hip_rope_args& a) {
         if (a.block_table) {
             if (a.block_size == 0) return GRANITE_HIP_EINVAL;
             if (a.positions && a.max_blocks_per_seq == 0) return GRANITE_HIP_EINVAL;
+            // One run of positions through one table: a table the caller declares too short
+            // would be read past its end (with per-token positions the kernel checks itself).
+            if (!a.positions && a.max_blocks_per_seq > 0 &&
+                (uint64_t(a.start_pos) + a.seq_len + a.block_size - 1) / a.block_size > a.max_blocks_per_seq)
+                return GRANITE_HIP_EOVERFLOW;
         } else if (!a.positions && uint64_t(a.start_pos) + a.seq_len > a.max_seq_len) {
             return GRANITE_HIP_EOVERFLOW;
         }

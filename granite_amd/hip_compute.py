@@ -207,20 +207,35 @@ class HipCompute:
     def decode_attention(self, *, q, q_dtype, k_cache, v_cache, out, batch_size, num_heads,
                          num_kv_heads, head_dim, scale, block_tables=None, seq_lens=None,
                          lse=None, block_size=0, max_blocks_per_seq=0, max_seq=0,
-                         fixed_seq_len=0, chunk_tokens=0) -> None:
+                         fixed_seq_len=0, chunk_tokens=0, workspace=None, workspace_bytes=None,
+                         query_workspace=False):
+        """workspace: a DeviceBuffer (or pointer + workspace_bytes) the launch takes its scratch
+        from instead of the library's buffer.  query_workspace: launch nothing, return the
+        scratch bytes the launch would need."""
         a = DecodeArgs(q=_p(q), q_dtype=q_dtype, k_cache=_p(k_cache), v_cache=_p(v_cache),
                        block_tables=_p(block_tables), seq_lens=_p(seq_lens), out=_p(out),
                        lse=_p(lse), batch_size=batch_size, num_heads=num_heads,
                        num_kv_heads=num_kv_heads, head_dim=head_dim, block_size=block_size,
                        max_blocks_per_seq=max_blocks_per_seq, max_seq=max_seq, scale=scale,
                        fixed_seq_len=fixed_seq_len, chunk_tokens=chunk_tokens)
-        check(self.lib.granite_hip_decode_attention(C.byref(a)), "decode_attention")
+        if query_workspace:
+            need = C.c_size_t()
+            check(self.lib.granite_hip_decode_workspace_required(C.byref(a), C.byref(need)),
+                  "decode_workspace_required")
+            return need.value
+        if workspace is not None:
+            nbytes = workspace.nbytes if workspace_bytes is None else workspace_bytes
+            check(self.lib.granite_hip_decode_attention_ws(C.byref(a), _p(workspace), nbytes),
+                  "decode_attention_ws")
+        else:
+            check(self.lib.granite_hip_decode_attention(C.byref(a)), "decode_attention")
 
     def attention(self, *, q, q_dtype, q_tok_stride, q_head_stride, out, out_dtype,
                   out_tok_stride, out_head_stride, seq_q, num_heads, num_kv_heads, head_dim, scale,
                   k_cache=None, v_cache=None, cache_len=0, max_seq=0, block_table=None,
                   block_size=0, k_extra=None, v_extra=None, extra_len=0, parents=None,
-                  mask_mode=MASK_CAUSAL, start_pos=0, lse=None) -> None:
+                  mask_mode=MASK_CAUSAL, start_pos=0, lse=None, workspace=None, workspace_bytes=None,
+                  query_workspace=False):
         a = AttentionArgs(q=_p(q), q_dtype=q_dtype, q_tok_stride=q_tok_stride,
                           q_head_stride=q_head_stride, out=_p(out), out_dtype=out_dtype,
                           out_tok_stride=out_tok_stride, out_head_stride=out_head_stride,
@@ -230,7 +245,24 @@ class HipCompute:
                           extra_len=extra_len, parents=_p(parents), mask_mode=mask_mode,
                           start_pos=start_pos, seq_q=seq_q, num_heads=num_heads,
                           num_kv_heads=num_kv_heads, head_dim=head_dim, scale=scale)
-        check(self.lib.granite_hip_attention(C.byref(a)), "attention")
+        if query_workspace:
+            need = C.c_size_t()
+            check(self.lib.granite_hip_attention_workspace_required(C.byref(a), C.byref(need)),
+                  "attention_workspace_required")
+            return need.value
+        if workspace is not None:
+            nbytes = workspace.nbytes if workspace_bytes is None else workspace_bytes
+            check(self.lib.granite_hip_attention_ws(C.byref(a), _p(workspace), nbytes), "attention_ws")
+        else:
+            check(self.lib.granite_hip_attention(C.byref(a)), "attention")
+
+    # ---- scratch memory
+    def workspace_bytes(self) -> int:
+        return int(self.lib.granite_hip_workspace_bytes())
+
+    def reserve_workspace(self, nbytes: int) -> None:
+        """Grow the library's scratch now, so that later launches needing no more never allocate."""
+        check(self.lib.granite_hip_reserve_workspace(nbytes), "reserve_workspace")
 
     def mfma_rate(self, operands, n_halves: int, iterations: int, shape: int = 32) -> float:
         """Launches the matrix-core rate kernel on `operands` (fp16 values); returns its flops."""

@@ -90,6 +90,20 @@ class HipCompute {
     // keys, causal / tree masks, optional log-sum-exp).
     Result<void> attention(const granite_hip_attention_args& args);
     Result<void> decode_attention(const granite_hip_decode_args& args);
+
+    // Scratch memory of the split-K launches.  MetalCompute's calls only enqueue
+    // (src/backend/metal/metal_compute.mm:150-207); here a launch that needs more scratch
+    // than the library holds waits for the device and reallocates, so a caller with a
+    // serving loop asks once what its largest launches need and reserves it up front,
+    // or passes a buffer of its own to the *_ws forms, which never allocate.
+    size_t workspace_bytes() const;
+    Result<void> reserve_workspace(size_t bytes);
+    Result<size_t> attention_workspace_required(const granite_hip_attention_args& args);
+    Result<size_t> decode_workspace_required(const granite_hip_decode_args& args);
+    Result<void> attention_ws(const granite_hip_attention_args& args, HipBuffer* workspace,
+                              size_t workspace_bytes);
+    Result<void> decode_attention_ws(const granite_hip_decode_args& args, HipBuffer* workspace,
+                                     size_t workspace_bytes);
 };
 
 // Process-wide instance, initialised on first use; nullptr when the GPU

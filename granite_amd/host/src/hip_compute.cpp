@@ -18,6 +18,7 @@ Result<void> hip_status_to_result(int status, const char* what) {
         case GRANITE_HIP_EUNSUPPORTED: code = ErrorCode::NotImplemented; break;
         case GRANITE_HIP_ENULL: code = ErrorCode::NullPointer; break;
         case GRANITE_HIP_EOVERFLOW: code = ErrorCode::InvalidArgument; break;  // kv_cache.cpp:61-65
+        case GRANITE_HIP_ESCRATCH: code = ErrorCode::InvalidArgument; break;
         default: code = ErrorCode::ExecutionFailed; break;                     // a hipError_t
     }
     return Error(code, std::string(what) + ": " + granite_hip_error_string(status));
@@ -166,6 +167,29 @@ Result<void> HipCompute::attention(const granite_hip_attention_args& args) {
 }
 Result<void> HipCompute::decode_attention(const granite_hip_decode_args& args) {
     return HIP_CALL(granite_hip_decode_attention(&args));
+}
+
+size_t HipCompute::workspace_bytes() const { return granite_hip_workspace_bytes(); }
+Result<void> HipCompute::reserve_workspace(size_t bytes) {
+    return HIP_CALL(granite_hip_reserve_workspace(bytes));
+}
+Result<size_t> HipCompute::attention_workspace_required(const granite_hip_attention_args& args) {
+    size_t bytes = 0;
+    GRANITE_TRY(HIP_CALL(granite_hip_attention_workspace_required(&args, &bytes)));
+    return bytes;
+}
+Result<size_t> HipCompute::decode_workspace_required(const granite_hip_decode_args& args) {
+    size_t bytes = 0;
+    GRANITE_TRY(HIP_CALL(granite_hip_decode_workspace_required(&args, &bytes)));
+    return bytes;
+}
+Result<void> HipCompute::attention_ws(const granite_hip_attention_args& args, HipBuffer* workspace,
+                                      size_t workspace_bytes) {
+    return HIP_CALL(granite_hip_attention_ws(&args, workspace, workspace_bytes));
+}
+Result<void> HipCompute::decode_attention_ws(const granite_hip_decode_args& args,
+                                             HipBuffer* workspace, size_t workspace_bytes) {
+    return HIP_CALL(granite_hip_decode_attention_ws(&args, workspace, workspace_bytes));
 }
 
 HipCompute* get_hip_compute() {

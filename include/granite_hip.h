@@ -18,8 +18,9 @@
  *     return immediately; results are valid after granite_hip_sync(), exactly
  *     like MetalCompute::sync() (src/backend/metal/metal_compute.mm:150-207);
  *   - "half" means IEEE binary16 stored as uint16_t;
- *   - head_dim must be 128 for the attention entry points (InvalidArgument
- *     otherwise, mirroring metal_compute.mm:2556-2559); the KV append/gather
+ *   - head_dim must be 128 for the attention entry points
+ *     (GRANITE_HIP_EUNSUPPORTED otherwise; the reference rejects head sizes it
+ *     has no kernel for, metal_compute.mm:2556-2559); the KV append/gather
  *     entry points accept any head_dim that is a multiple of 8.
  *
  * Layouts (D = head_dim, G = num_heads / num_kv_heads)
@@ -46,6 +47,7 @@ extern "C" {
 #define GRANITE_HIP_EUNSUPPORTED (-4)/* ErrorCode::NotImplemented */
 #define GRANITE_HIP_ENULL (-5)       /* ErrorCode::NullPointer */
 #define GRANITE_HIP_EOVERFLOW (-6)   /* KV cache overflow (kv_cache.cpp:61-65) */
+#define GRANITE_HIP_ESCRATCH (-7)    /* the scratch buffer given is too small for this launch */
 
 /* element types of Q / output tensors */
 #define GRANITE_HIP_F32 0
@@ -98,7 +100,11 @@ int granite_hip_memcpy_d2d(void *dst, const void *src, size_t bytes);
 int granite_hip_memset(void *dst, int value, size_t bytes);
 int granite_hip_sync(void);
 /* Use `stream` (a hipStream_t) for all later launches; NULL restores the
- * library's own stream. */
+ * library's own stream.  The hand-over is ordered: the new stream first waits
+ * for everything queued on the old one, because all launches share one
+ * scratch buffer.  Launches are single-threaded and go to one stream at a
+ * time, like the one command queue of MetalCompute
+ * (src/backend/metal/metal_compute.mm:150-207); the library takes no lock. */
 int granite_hip_set_stream(void *stream);
 void *granite_hip_get_stream(void);
 
@@ -357,7 +363,12 @@ int granite_hip_rope_multihead(void *q, void *k, uint32_t num_heads_q, uint32_t 
  *                 device, so the kernel does: a token whose position is
  *                 negative or beyond the cos/sin tables is left untouched, one
  *                 whose position is beyond its cache (max_seq_len, or
- *                 max_blocks_per_seq blocks) is rotated but not stored. */
+ *                 max_blocks_per_seq blocks) is rotated but not stored.
+ *   max_blocks_per_seq  entries the block table holds (per sequence).  Without
+ *                 positions, 0 means "not stated" (as in
+ *                 MetalCompute::paged_kv_cache_append, which takes no bound);
+ *                 otherwise start_pos + seq_len tokens must fit that many
+ *                 blocks, or the call fails with GRANITE_HIP_EOVERFLOW. */
 typedef struct granite_hip_rope_args {
     void *q;
     void *q_f16;
@@ -394,8 +405,39 @@ int granite_hip_rope_append(const granite_hip_rope_args *args);
 int granite_hip_mfma_rate(const void *operands_f16, uint64_t n_halves, uint32_t iterations,
                           int shape, double *flops);
 
-/* Bytes of device scratch the library keeps for split-K partial results. */
+/* ---- scratch memory ------------------------------------------------------ *
+ * Decode and prefill launches that split the keys over several workgroups
+ * keep partial results (and the stream decode kernel its plan, large trees
+ * their ancestor mask) in device scratch.  By default that is one buffer the
+ * library owns and grows on demand; growing waits for the device, frees and
+ * allocates, so a first call with a larger shape stalls.  MetalCompute's calls
+ * only ever enqueue (src/backend/metal/metal_compute.mm:150-207); to get the
+ * same here either reserve once, up front, what the largest launch will need,
+ * or hand every launch its own scratch with the _ws forms, which never
+ * allocate and never synchronise. */
+
+/* Bytes of device scratch the library holds at the moment. */
 size_t granite_hip_workspace_bytes(void);
+
+/* Grows the library's scratch to at least `bytes` now (waits for the device
+ * when it has to grow).  Later launches that need no more never allocate. */
+int granite_hip_reserve_workspace(size_t bytes);
+
+/* Scratch bytes the launch described by `args` needs (0 for shapes that need
+ * none).  Nothing is launched; pointers in `args` are only tested for NULL. */
+int granite_hip_decode_workspace_required(const granite_hip_decode_args *args, size_t *bytes);
+int granite_hip_attention_workspace_required(const granite_hip_attention_args *args,
+                                             size_t *bytes);
+
+/* granite_hip_decode_attention / granite_hip_attention with caller-owned
+ * scratch: `workspace` (256-byte aligned device memory of `workspace_bytes`)
+ * is the only scratch the launch uses, and it stays in use until the launch
+ * has run.  Too small -> GRANITE_HIP_ESCRATCH, nothing launched.  workspace
+ * NULL: the library's buffer, as in the plain forms. */
+int granite_hip_decode_attention_ws(const granite_hip_decode_args *args, void *workspace,
+                                    size_t workspace_bytes);
+int granite_hip_attention_ws(const granite_hip_attention_args *args, void *workspace,
+                             size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

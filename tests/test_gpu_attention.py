@@ -41,7 +41,7 @@ def test_causal_prefill_small(gpu, oracle, seq, hq, hkv, max_seq, q_dtype, out_d
     want, want_lse = oracle.attention_cached(q32[None], case.k_cache, case.v_cache, seq, 0, case.scale)
     got, got_lse = _prefill(gpu, q32 if q_dtype == F32 else case.q, case.k_cache, case.v_cache, seq, seq, 0, hq,
                             hkv, max_seq, case.scale, q_dtype, out_dtype)
-    assert_close(got, want[0], "out", abs_tol=2e-3 if out_dtype == F32 else 3e-3)
+    assert_close(got, want[0], "out")
     assert_lse(got_lse, want_lse[0], "lse")
     # query 0 sees only key 0: the output row is V[0] (up to the final 1/l multiply)
     for h in range(hq):
@@ -54,15 +54,11 @@ def test_causal_prefill_config(gpu, oracle):
     say("prefill config seq=2048")
     got, got_lse = _prefill(gpu, case.q, case.k_cache, case.v_cache, 2048, 2048, 0, 32, 8, 2048, case.scale, F16,
                             F16)
-    # oracle on a sample of query rows (the full pass is 34 GFLOP of scalar code)
-    k = np.transpose(case.k_cache, (1, 0, 2)).astype(np.float32)
-    v = np.transpose(case.v_cache, (1, 0, 2)).astype(np.float32)
-    rows = [0, 1, 63, 64, 127, 128, 1000, 1023, 1024, 2000, 2047]
-    for r in rows:
-        want, want_lse = oracle.attention_core(case.q[None, r:r + 1].astype(np.float32), k[:r + 1], v[:r + 1], r,
-                                               case.scale)
-        assert_close(got[r], want[0, 0], f"row {r}", abs_tol=3e-3)
-        assert_lse(got_lse[:, r], want_lse[0, :, 0], f"lse row {r}")
+    # every one of the 2048 rows against the oracle (34 GFLOP of scalar code: seconds)
+    want, want_lse = oracle.attention_cached(case.q[None].astype(np.float32), case.k_cache, case.v_cache, 2048, 0,
+                                             case.scale)
+    assert_close(got, want[0], "out")
+    assert_lse(got_lse, want_lse[0], "lse")
 
 
 def test_reference_entry_point_multihead_attention(gpu, oracle):
@@ -105,7 +101,7 @@ def test_chunked_prefill_over_paged_cache_small(gpu, oracle, prefix, chunk, bs, 
                   num_kv_heads=hkv, head_dim=128, scale=case.scale, k_cache=dk, v_cache=dv, cache_len=total,
                   block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
     gpu.sync()
-    assert_close(out.read(np.float16, (chunk, hq, 128)).astype(np.float32), want[0], "out", abs_tol=3e-3)
+    assert_close(out.read(np.float16, (chunk, hq, 128)).astype(np.float32), want[0], "out")
     assert_lse(lse.read(np.float32, (hq, chunk)), want_lse[0], "lse")
 
 
@@ -141,13 +137,14 @@ def test_chunked_prefill_random_shapes(gpu, oracle, trial):
                   cache_len=total, block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
     gpu.sync()
     got = out.read(np.float32 if f32 else np.float16, (chunk, hq, 128)).astype(np.float32)
-    assert_close(got, want[0], "out", abs_tol=3e-3)
+    assert_close(got, want[0], "out")
     assert_lse(lse.read(np.float32, (hq, chunk)), want_lse[0], "lse")
 
 
 def test_chunked_prefill_config(gpu, oracle):
     """32768-token paged prefix (block 32), 512-token chunk, 64 q heads, 8 KV
-    heads, values 0.5*N(0,1); append bit-exact, attention on sampled rows."""
+    heads, values 0.5*N(0,1); append bit-exact, attention on every 8th row and the
+    rows at the run edges."""
     case = W.make_chunked_prefill()
     say("chunked prefill config prefix=32768 chunk=512")
     hq, hkv, bs, prefix, chunk = 64, 8, 32, case.prefix_len, case.chunk
@@ -174,10 +171,13 @@ def test_chunked_prefill_config(gpu, oracle):
     got = out.read(np.float16, (chunk, hq, 128)).astype(np.float32)
     got_lse = lse.read(np.float32, (hq, chunk))
     k32, v32 = k_all.astype(np.float32), v_all.astype(np.float32)
-    for r in (0, 1, 31, 255, 511):
+    # every 8th row, the rows either side of the 128-row run edges and of the seam where the
+    # paired runs of a workgroup meet, and the first and last row of the chunk
+    rows = sorted(set(range(0, chunk, 8)) | {1, 31, 127, 128, 129, 255, 256, 257, 383, 384, 385, 510, 511})
+    for r in rows:
         want, want_lse = oracle.attention_core(case.q[None, r:r + 1].astype(np.float32), k32[:prefix + r + 1],
                                                v32[:prefix + r + 1], prefix + r, case.scale)
-        assert_close(got[r], want[0, 0], f"row {r}", abs_tol=3e-3)
+        assert_close(got[r], want[0, 0], f"row {r}")
         assert_lse(got_lse[:, r], want_lse[0, :, 0], f"lse row {r}")
 
 
@@ -303,7 +303,7 @@ def test_attention_rejects_bad_arguments(gpu):
     base = dict(q=buf, q_dtype=F32, q_tok_stride=1024, q_head_stride=128, out=buf, out_dtype=F32,
                 out_tok_stride=1024, out_head_stride=128, seq_q=4, num_heads=8, num_kv_heads=2, head_dim=128,
                 scale=0.1, k_cache=buf, v_cache=buf, cache_len=4, max_seq=8, mask_mode=MASK_CAUSAL)
-    for bad, code in ((dict(head_dim=64), _capi.EINVAL), (dict(num_kv_heads=3), _capi.EINVAL),
+    for bad, code in ((dict(head_dim=64), _capi.EUNSUPPORTED), (dict(num_kv_heads=3), _capi.EINVAL),
                       (dict(out=None), _capi.ENULL), (dict(max_seq=2), _capi.EINVAL),
                       (dict(mask_mode=9), _capi.EINVAL), (dict(q_tok_stride=1022), _capi.EINVAL),
                       (dict(mask_mode=MASK_TREE), _capi.ENULL), (dict(cache_len=0), _capi.EINVAL),

@@ -194,7 +194,7 @@ def test_decode_rejects_bad_arguments(gpu):
     buf = dev(np.zeros(4096, np.float32))
     base = dict(q=buf, q_dtype=F32, k_cache=buf, v_cache=buf, out=buf, batch_size=1, num_heads=8,
                 num_kv_heads=2, head_dim=128, scale=0.1, max_seq=16, fixed_seq_len=4)
-    for bad, code in ((dict(head_dim=64), _capi.EINVAL), (dict(num_kv_heads=3), _capi.EINVAL),
+    for bad, code in ((dict(head_dim=64), _capi.EUNSUPPORTED), (dict(num_kv_heads=3), _capi.EINVAL),
                       (dict(q=None), _capi.ENULL), (dict(fixed_seq_len=0), _capi.EINVAL),
                       (dict(fixed_seq_len=17), _capi.EINVAL), (dict(chunk_tokens=48), _capi.EINVAL),
                       (dict(q_dtype=7), _capi.EINVAL)):
