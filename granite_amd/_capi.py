@@ -180,6 +180,8 @@ SIGNATURES = {
     "granite_hip_attention_workspace_required": (_int, [C.POINTER(AttentionArgs), C.POINTER(C.c_size_t)]),
     "granite_hip_decode_attention_ws": (_int, [C.POINTER(DecodeArgs), _vp, C.c_size_t]),
     "granite_hip_attention_ws": (_int, [C.POINTER(AttentionArgs), _vp, C.c_size_t]),
+    "granite_hip_decode_attention_static": (_int, [C.POINTER(DecodeArgs)]),
+    "granite_hip_static_scratch_bytes": (C.c_size_t, []),
 }
 
 _lib = None

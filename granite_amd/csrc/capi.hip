@@ -11,7 +11,19 @@
 
 #include "common.h"
 
+// Scratch memory of granite_hip_decode_attention_static, the entry point for callers
+// that cannot allocate.  One copy per device, held until the process ends.  In host code
+// this name is only a handle for hipGetSymbolAddress: the address kernels and copies use
+// is the one resolved per device in granite_hip_init.
+static constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace ghip {
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};  // device address of `scratch`, per device
+}  // namespace
 
 Context& ctx() {
     static Context c;
@@ -63,6 +75,7 @@ struct PendingTiming {
 };
 struct TimingState {
     bool enabled = false;
+    bool suppressed = false;  // inside an entry point that must not create events
     std::vector<PendingTiming> pending;
     std::vector<hipEvent_t> free_events;
     std::map<std::string, std::pair<double, uint64_t>> stats;
@@ -101,8 +114,11 @@ void resolve_timings() {
 }
 }  // namespace
 
+TimingSuppressed::TimingSuppressed() : was_(timing().suppressed) { timing().suppressed = true; }
+TimingSuppressed::~TimingSuppressed() { timing().suppressed = was_; }
+
 KernelTimerScope::KernelTimerScope(const char* name) : name_(name) {
-    if (!timing().enabled) return;
+    if (!timing().enabled || timing().suppressed) return;
     start_ = take_event();
     if (start_) (void)hipEventRecord(start_, ctx().stream);
 }
@@ -155,6 +171,14 @@ int granite_hip_init(int device) {
         std::fprintf(stderr, "granite_hip: device %d is %s; this library holds gfx950 code only\n",
                      device, prop.gcnArchName);
         return GRANITE_HIP_EUNSUPPORTED;
+    }
+    if (device >= ghip::kMaxDevices) return GRANITE_HIP_EINVAL;
+    if (!ghip::g_static_scratch[device]) {
+        // every device holds its own copy of the array at its own address
+        void* ptr = nullptr;
+        GHIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr || (reinterpret_cast<uintptr_t>(ptr) & 255)) return GRANITE_HIP_EINVAL;
+        ghip::g_static_scratch[device] = ptr;
     }
     GHIP_CHECK(hipStreamCreateWithFlags(&c.own_stream, hipStreamNonBlocking));
     c.stream = c.own_stream;
@@ -407,6 +431,20 @@ int granite_hip_decode_attention_ws(const granite_hip_decode_args* args, void* w
     ghip::ScratchSource src;
     src.fixed = workspace;
     src.fixed_bytes = workspace_bytes;
+    return ghip::launch_decode(*args, src);
+}
+
+size_t granite_hip_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int granite_hip_decode_attention_static(const granite_hip_decode_args* args) {
+    GHIP_REQUIRE_INIT();
+    if (!args) return GRANITE_HIP_ENULL;
+    ghip::ScratchSource src;
+    src.fixed = ghip::g_static_scratch[ctx().device];
+    src.fixed_bytes = kStaticScratchBytes;
+    if (!src.fixed) return GRANITE_HIP_ENOTINIT;
+    // no events either: per-kernel timing creates them on demand
+    ghip::TimingSuppressed quiet;
     return ghip::launch_decode(*args, src);
 }
 

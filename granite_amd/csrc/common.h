@@ -72,6 +72,17 @@ struct KernelTimerScope {
     hipEvent_t start_ = nullptr;
 };
 
+// While one of these lives, KernelTimerScope records nothing (and so creates no events).
+struct TimingSuppressed {
+    TimingSuppressed();
+    ~TimingSuppressed();
+    TimingSuppressed(const TimingSuppressed&) = delete;
+    TimingSuppressed& operator=(const TimingSuppressed&) = delete;
+
+  private:
+    bool was_;
+};
+
 inline int launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? GRANITE_HIP_OK : static_cast<int>(e);

@@ -208,7 +208,7 @@ class HipCompute:
                          num_kv_heads, head_dim, scale, block_tables=None, seq_lens=None,
                          lse=None, block_size=0, max_blocks_per_seq=0, max_seq=0,
                          fixed_seq_len=0, chunk_tokens=0, workspace=None, workspace_bytes=None,
-                         query_workspace=False):
+                         query_workspace=False, static_scratch=False):
         """workspace: a DeviceBuffer (or pointer + workspace_bytes) the launch takes its scratch
         from instead of the library's buffer.  query_workspace: launch nothing, return the
         scratch bytes the launch would need."""
@@ -223,6 +223,9 @@ class HipCompute:
             check(self.lib.granite_hip_decode_workspace_required(C.byref(a), C.byref(need)),
                   "decode_workspace_required")
             return need.value
+        if static_scratch:  # the entry point that allocates nothing
+            check(self.lib.granite_hip_decode_attention_static(C.byref(a)), "decode_attention_static")
+            return None
         if workspace is not None:
             nbytes = workspace.nbytes if workspace_bytes is None else workspace_bytes
             check(self.lib.granite_hip_decode_attention_ws(C.byref(a), _p(workspace), nbytes),

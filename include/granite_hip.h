@@ -439,6 +439,23 @@ int granite_hip_decode_attention_ws(const granite_hip_decode_args *args, void *w
 int granite_hip_attention_ws(const granite_hip_attention_args *args, void *workspace,
                              size_t workspace_bytes);
 
+/* granite_hip_decode_attention for callers that cannot allocate.  It has no
+ * counterpart in the reference; it is for code under HIP graph capture, tight
+ * serving loops and harnesses that forbid hipMalloc.  Same arguments, same
+ * kernels and bit-identical results, but the scratch (the stream kernel's
+ * plan and partial results) is a fixed array in device memory that the library
+ * holds on every GPU it runs on, granite_hip_static_scratch_bytes() (32 MiB)
+ * long, and the call makes no allocation of any kind: no hipMalloc, no
+ * hipFree, no events (per-kernel timing skips these launches).  A launch that
+ * needs more -- granite_hip_decode_workspace_required() tells -- fails with
+ * GRANITE_HIP_ESCRATCH and launches nothing.  Every call on a GPU uses that
+ * GPU's one array: calls that overlap on one GPU (two streams, two threads)
+ * race; calls queued on the library's single stream are ordered and safe.
+ * Nothing in the array has to start at zero, the kernels write every partial
+ * they later read. */
+int granite_hip_decode_attention_static(const granite_hip_decode_args *args);
+size_t granite_hip_static_scratch_bytes(void);
+
 #ifdef __cplusplus
 }
 #endif
