@@ -7,6 +7,7 @@
 #include <random>
 
 #include "check.h"
+#include "granite/chunked_prefill.h"
 #include "granite/hip_backend.h"
 #include "granite/hip_compute.h"
 #include "granite/kv_cache.h"
@@ -24,6 +25,12 @@ int go_kv_cache_append_f16(uint16_t* cache, const uint16_t* src, int num_kv_head
 void go_paged_kv_cache_append_f32(uint16_t* pool, const float* src, const int32_t* table,
                                   int num_kv_heads, int head_dim, int start_pos, int new_len,
                                   int block_size);
+int go_kv_cache_append_f32(uint16_t* cache, const float* src, int num_kv_heads, int head_dim,
+                           int current_len, int new_len, int max_seq);
+void go_attention_paged(const float* q, const uint16_t* pool_k, const uint16_t* pool_v,
+                        const int32_t* table, int block_size, float* context, float* lse, int batch,
+                        int seq_len, int num_heads, int num_kv_heads, int head_dim, int total_seq,
+                        int start_pos, float scale);
 void go_attention_cached(const float* q, const uint16_t* cache_k, const uint16_t* cache_v,
                          float* context, float* lse, int batch, int seq_len, int num_heads,
                          int num_kv_heads, int head_dim, int total_seq, int max_seq,
@@ -719,6 +726,200 @@ TEST_CASE(paged_prefill_then_batched_decode_steps) {
     }
     CHECK_CODE(step.begin_step(std::span<const int>(slots, 0)), ErrorCode::InvalidArgument);
 }
+
+// The chunk loop of forward_prefill_raw (src/llm/transformer.mm:3467-3477, 3681-3866) on the
+// host layer: a 2048-token prompt fed in chunks of 512 and of 96 (ragged last chunk), then a
+// second prompt behind it in chunks of 128, into a paged sequence; and a prompt into a
+// contiguous KVCache.  Every chunk's rotated Q/K, the caches and the outputs are compared
+// with the oracle's one-shot pass over the whole prompt: rotation and cache rows bit for bit
+// (truncating conversion), outputs within the attention tolerance.
+TEST_CASE(chunked_prefill_driver) {
+    REQUIRE(backend() != nullptr);
+    CHECK(prefill_chunk_tokens(2048, 0) == 2048);       // no chunking asked for
+    CHECK(prefill_chunk_tokens(2048, 4096) == 2048);    // chunk not below the prompt
+    CHECK(prefill_chunk_tokens(2048, 512) == 512);
+    CHECK(prefill_chunk_tokens(2048, 7) == 32);         // raised to the minimum of 32
+    CHECK(prefill_chunk_tokens(20, 7) == 20);           // 32 capped by the prompt
+    const int hq = 8, hkv = 2, bs = 16, layers = 2;
+    const int max_pos = 2560;
+    const float scale = 1.0f / std::sqrt(float(D));
+    RoPECache rope;
+    rope.initialize(max_pos, D, 10000.0f);
+    std::vector<float> cos_t(size_t(max_pos) * D / 2), sin_t(cos_t.size());
+    go_rope_table(cos_t.data(), sin_t.data(), max_pos, D, 10000.0f);
+
+    auto transpose_heads = [&](const std::vector<float>& x, int n) {  // [n, hkv, D] -> [hkv, n, D]
+        std::vector<float> t(x.size());
+        for (int s = 0; s < n; ++s)
+            for (int h = 0; h < hkv; ++h)
+                std::memcpy(&t[(size_t(h) * n + s) * D], &x[(size_t(s) * hkv + h) * D], D * sizeof(float));
+        return t;
+    };
+
+    // ---- paged sequence
+    ModelConfig cfg;
+    cfg.num_layers = layers;
+    cfg.num_heads = hq;
+    cfg.num_kv_heads = hkv;
+    cfg.head_dim = D;
+    PagedKVPool pool;
+    REQUIRE(pool.initialize(cfg, 2, 170 * bs, bs, backend()).ok());
+    BlockManager& mgr = pool.block_manager();
+    const int slot = pool.acquire_slot();
+    REQUIRE(slot >= 0);
+    PagedKVCache& seq = pool.get_cache(slot);
+    // a few blocks taken and given back first, so that the table is not the identity
+    {
+        PagedKVCache other(&mgr);
+        REQUIRE(other.append_tokens(5 * bs));
+        REQUIRE(seq.append_tokens(1));
+        other.release();
+        seq.truncate(0);
+    }
+    std::vector<std::vector<uint16_t>> want_k, want_v;
+    for (int l = 0; l < layers; ++l) {
+        want_k.push_back(download<uint16_t>(mgr.k_cache(l)));
+        want_v.push_back(download<uint16_t>(mgr.v_cache(l)));
+    }
+    ChunkedPrefill driver;
+    CHECK_CODE(driver.begin(10, 0), ErrorCode::InvalidState);
+    REQUIRE(driver.initialize(&seq, 160, backend()).ok());
+    driver.set_rounding(GRANITE_HIP_ROUND_TRUNCATE);
+    CHECK_CODE(driver.begin(161 * bs, 512), ErrorCode::InvalidArgument);  // beyond the block table
+    CHECK(seq.seq_len() == 0);
+
+    struct Prompt {
+        int tokens;
+        uint32_t chunk_size;
+        int expect_chunks;
+    };
+    uint32_t seed = 9100;
+    int held = 0;
+    for (const Prompt pr : {Prompt{2048, 512, 4}, Prompt{300, 128, 3}}) {
+        REQUIRE(driver.begin(pr.tokens, pr.chunk_size).ok());
+        CHECK(driver.num_chunks() == pr.expect_chunks);
+        CHECK(driver.base_len() == held);
+        CHECK(seq.seq_len() == held + pr.tokens);
+        std::vector<int32_t> table(seq.block_table().begin(), seq.block_table().end());
+        for (int l = 0; l < layers; ++l) {
+            const int n = pr.tokens;
+            auto q = randn(size_t(n) * hq * D, seed++), k = randn(size_t(n) * hkv * D, seed++),
+                 v = randn(size_t(n) * hkv * D, seed++);
+            Tensor Q = upload({n, hq, D}, DataType::FP32, q);
+            Tensor K = upload({n, hkv, D}, DataType::FP32, k);
+            Tensor V = upload({n, hkv, D}, DataType::FP32, v);
+            Tensor O = Tensor::allocate({n, hq, D}, DataType::FP32, backend()).take();
+            if (l == 0) {
+                CHECK_OK(driver.run_layer(l, Q, K, V, O, scale, &rope));
+            } else {  // chunk by chunk through run_chunk, on tensors of the chunk's own
+                for (int c = 0; c < driver.num_chunks(); ++c) {
+                    const int s0 = driver.chunk_start(c), len = driver.chunk_len(c);
+                    auto part = [&](Tensor& t) { return t.slice(0, s0, s0 + len).take(); };
+                    Tensor qc = part(Q), kc = part(K), vc = part(V), oc = part(O);
+                    CHECK_OK(driver.run_chunk(l, c, qc, kc, vc, oc, scale, &rope));
+                }
+            }
+            // oracle: the whole prompt at once
+            CHECK(go_rope_apply(q.data(), n, hq, D, held, cos_t.data(), sin_t.data(), max_pos) == 0);
+            CHECK(go_rope_apply(k.data(), n, hkv, D, held, cos_t.data(), sin_t.data(), max_pos) == 0);
+            go_paged_kv_cache_append_f32(want_k[l].data(), transpose_heads(k, n).data(), table.data(), hkv, D,
+                                         held, n, bs);
+            go_paged_kv_cache_append_f32(want_v[l].data(), transpose_heads(v, n).data(), table.data(), hkv, D,
+                                         held, n, bs);
+            std::vector<float> want(q.size());
+            go_attention_paged(q.data(), want_k[l].data(), want_v[l].data(), table.data(), bs, want.data(),
+                               nullptr, 1, n, hq, hkv, D, held + n, held, scale);
+            CHECK(download<float>(Q) == q);  // rotated at the right positions: the oracle's bits
+            CHECK(download<float>(K) == k);
+            CHECK(download<uint16_t>(mgr.k_cache(l)) == want_k[l]);
+            CHECK(download<uint16_t>(mgr.v_cache(l)) == want_v[l]);
+            CHECK(close_enough(download<float>(O), want, "chunked prefill, paged"));
+            for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+        }
+        driver.finish();
+        held += pr.tokens;
+        CHECK(seq.seq_len() == held);
+    }
+    // the same 2048-token prompt again in chunks of 96 (22 chunks, the last of 32) into a
+    // fresh sequence: identical pools row for row, outputs within tolerance of the oracle's
+    {
+        const int slot2 = pool.acquire_slot();
+        REQUIRE(slot2 >= 0);
+        PagedKVCache& seq2 = pool.get_cache(slot2);
+        // not enough blocks left for 2048 tokens: begin() fails and gives everything back
+        ChunkedPrefill d2;
+        REQUIRE(d2.initialize(&seq2, 160, backend()).ok());
+        const int free_before = pool.num_free_blocks();
+        CHECK_CODE(d2.begin(2048, 96), ErrorCode::AllocationFailed);
+        CHECK(seq2.seq_len() == 0 && pool.num_free_blocks() == free_before);
+        seq.release();
+        REQUIRE(d2.begin(2048, 96).ok());
+        d2.set_rounding(GRANITE_HIP_ROUND_TRUNCATE);
+        CHECK(d2.num_chunks() == 22 && d2.chunk_len(21) == 32 && d2.chunk_start(21) == 2016);
+        std::vector<int32_t> table(seq2.block_table().begin(), seq2.block_table().end());
+        const int n = 2048;
+        auto q = randn(size_t(n) * hq * D, seed++), k = randn(size_t(n) * hkv * D, seed++),
+             v = randn(size_t(n) * hkv * D, seed++);
+        Tensor Q = upload({n, hq, D}, DataType::FP32, q);
+        Tensor K = upload({n, hkv, D}, DataType::FP32, k);
+        Tensor V = upload({n, hkv, D}, DataType::FP32, v);
+        Tensor O = Tensor::allocate({n, hq, D}, DataType::FP32, backend()).take();
+        CHECK_OK(d2.run_layer(0, Q, K, V, O, scale, &rope));
+        CHECK(go_rope_apply(q.data(), n, hq, D, 0, cos_t.data(), sin_t.data(), max_pos) == 0);
+        CHECK(go_rope_apply(k.data(), n, hkv, D, 0, cos_t.data(), sin_t.data(), max_pos) == 0);
+        auto pk = download<uint16_t>(mgr.k_cache(0)), pv = download<uint16_t>(mgr.v_cache(0));
+        auto wk = want_k[0], wv = want_v[0];
+        go_paged_kv_cache_append_f32(wk.data(), transpose_heads(k, n).data(), table.data(), hkv, D, 0, n, bs);
+        go_paged_kv_cache_append_f32(wv.data(), transpose_heads(v, n).data(), table.data(), hkv, D, 0, n, bs);
+        CHECK(pk == wk);
+        CHECK(pv == wv);
+        std::vector<float> want(q.size());
+        go_attention_paged(q.data(), wk.data(), wv.data(), table.data(), bs, want.data(), nullptr, 1, n, hq, hkv,
+                           D, n, 0, scale);
+        CHECK(close_enough(download<float>(O), want, "chunked prefill, 22 chunks of 96"));
+        for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+    }
+
+    // ---- contiguous KVCache, as the reference's loop runs it
+    {
+        const int max_seq = 700, n = 600;
+        auto made = KVCache::allocate(cfg, max_seq, backend());
+        REQUIRE(made.ok());
+        KVCache cache = made.take();
+        ChunkedPrefill d3;
+        REQUIRE(d3.initialize(&cache, backend()).ok());
+        d3.set_rounding(GRANITE_HIP_ROUND_TRUNCATE);
+        CHECK_CODE(d3.begin(701, 256), ErrorCode::InvalidArgument);  // overflow (kv_cache.cpp:61-65)
+        REQUIRE(d3.begin(n, 256).ok());
+        CHECK(d3.num_chunks() == 3 && d3.chunk_len(2) == 88);
+        for (int l = 0; l < layers; ++l) {
+            auto q = randn(size_t(n) * hq * D, seed++), k = randn(size_t(n) * hkv * D, seed++),
+                 v = randn(size_t(n) * hkv * D, seed++);
+            Tensor Q = upload({n, hq, D}, DataType::FP32, q);
+            Tensor K = upload({n, hkv, D}, DataType::FP32, k);
+            Tensor V = upload({n, hkv, D}, DataType::FP32, v);
+            Tensor O = Tensor::allocate({n, hq, D}, DataType::FP32, backend()).take();
+            auto kv = cache.get(l);
+            auto ck = download<uint16_t>(kv.first), cv = download<uint16_t>(kv.second);
+            CHECK_OK(d3.run_layer(l, Q, K, V, O, scale, &rope));
+            CHECK(cache.seq_len() == 0);  // advances after the last layer only
+            CHECK(go_rope_apply(q.data(), n, hq, D, 0, cos_t.data(), sin_t.data(), max_pos) == 0);
+            CHECK(go_rope_apply(k.data(), n, hkv, D, 0, cos_t.data(), sin_t.data(), max_pos) == 0);
+            CHECK(go_kv_cache_append_f32(ck.data(), k.data(), hkv, D, 0, n, max_seq) == 0);
+            CHECK(go_kv_cache_append_f32(cv.data(), v.data(), hkv, D, 0, n, max_seq) == 0);
+            std::vector<float> want(q.size());
+            go_attention_cached(q.data(), ck.data(), cv.data(), want.data(), nullptr, 1, n, hq, hkv, D, n, max_seq,
+                                0, scale);
+            CHECK(download<uint16_t>(kv.first) == ck);
+            CHECK(download<uint16_t>(kv.second) == cv);
+            CHECK(close_enough(download<float>(O), want, "chunked prefill, contiguous cache"));
+            for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+        }
+        d3.finish();
+        CHECK(cache.seq_len() == n);
+    }
+}
+
 
 TEST_CASE(speculative_commit_of_accepted_path) {
     REQUIRE(backend() != nullptr);
