@@ -173,6 +173,11 @@ SIGNATURES = {
                                              _u32, _u32, _u32, _u32, _int]),
     "granite_hip_rope_multihead": (_int, [_vp, _vp, _u32, _u32, _u32, _u32, _u32, _f32]),
     "granite_hip_rope_append": (_int, [C.POINTER(RopeArgs)]),
+    "granite_hip_fused_qkv_matvec_q4k": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
+    "granite_hip_fused_qkv_matvec_q4k_batched": (
+        _int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _u32, _u32, _u32, _u32]),
+    "granite_hip_matvec_q4k": (_int, [_vp, _vp, _vp, _u32, _u32]),
+    "granite_hip_matvec_q4k_batched": (_int, [_vp, _i64, _vp, _vp, _i64, _u32, _u32, _u32]),
     "granite_hip_mfma_rate": (_int, [_vp, C.c_uint64, _u32, _int, C.POINTER(C.c_double)]),
     "granite_hip_workspace_bytes": (C.c_size_t, []),
     "granite_hip_reserve_workspace": (_int, [C.c_size_t]),

@@ -558,6 +558,40 @@ int granite_hip_paged_kv_gather(void* dst_k, void* dst_v, const void* k_cache,
                                         head_dim, len, block_size, max_seq_len);
 }
 
+// ---- projections on Q4_K weights ------------------------------------------------
+
+int granite_hip_fused_qkv_matvec_q4k_batched(const void* x, int64_t x_stride, const void* wq,
+                                             const void* wk, const void* wv, void* yq, void* yk,
+                                             void* yv, int64_t yq_stride, int64_t ykv_stride,
+                                             uint32_t K, uint32_t Nq, uint32_t Nkv, uint32_t batch) {
+    GHIP_REQUIRE_INIT();
+    const void* const w[3] = {wq, wk, wv};
+    void* const y[3] = {yq, yk, yv};
+    const int64_t ys[3] = {yq_stride, ykv_stride, ykv_stride};
+    const uint32_t n[3] = {Nq, Nkv, Nkv};
+    return ghip::launch_matvec_q4k(x, x_stride, w, y, ys, n, K, batch);
+}
+
+int granite_hip_fused_qkv_matvec_q4k(const void* x, const void* wq, const void* wk, const void* wv,
+                                     void* yq, void* yk, void* yv, uint32_t K, uint32_t Nq,
+                                     uint32_t Nkv) {
+    return granite_hip_fused_qkv_matvec_q4k_batched(x, K, wq, wk, wv, yq, yk, yv, Nq, Nkv, K, Nq, Nkv, 1);
+}
+
+int granite_hip_matvec_q4k_batched(const void* x, int64_t x_stride, const void* w, void* y,
+                                   int64_t y_stride, uint32_t K, uint32_t N, uint32_t batch) {
+    GHIP_REQUIRE_INIT();
+    const void* const ws[3] = {w, nullptr, nullptr};
+    void* const ys[3] = {y, nullptr, nullptr};
+    const int64_t strides[3] = {y_stride, 0, 0};
+    const uint32_t n[3] = {N, 0, 0};
+    return ghip::launch_matvec_q4k(x, x_stride, ws, ys, strides, n, K, batch);
+}
+
+int granite_hip_matvec_q4k(const void* x, const void* w, void* y, uint32_t K, uint32_t N) {
+    return granite_hip_matvec_q4k_batched(x, K, w, y, N, K, N, 1);
+}
+
 // ---- measurement aid ----------------------------------------------------------
 
 int granite_hip_mfma_rate(const void* operands_f16, uint64_t n_halves, uint32_t iterations,

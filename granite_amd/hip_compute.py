@@ -310,6 +310,28 @@ class HipCompute:
                      max_blocks_per_seq=max_blocks_per_seq)
         check(self.lib.granite_hip_rope_append(C.byref(a)), "rope_append")
 
+    # ---- projections on Q4_K weights
+    def fused_qkv_matvec_q4k(self, x, Wq, Wk, Wv, yq, yk, yv, K, Nq, Nkv, batch=1, x_stride=None,
+                             yq_stride=None, ykv_stride=None) -> None:
+        """MetalCompute::fused_qkv_matvec_q4k (include/granite/metal_compute.h:683-694): the
+        three attention projections of one token (or of `batch` tokens) in one launch."""
+        if batch == 1 and x_stride is None and yq_stride is None and ykv_stride is None:
+            check(self.lib.granite_hip_fused_qkv_matvec_q4k(_p(x), _p(Wq), _p(Wk), _p(Wv), _p(yq), _p(yk),
+                                                            _p(yv), K, Nq, Nkv), "fused_qkv_matvec_q4k")
+            return
+        check(self.lib.granite_hip_fused_qkv_matvec_q4k_batched(
+            _p(x), K if x_stride is None else x_stride, _p(Wq), _p(Wk), _p(Wv), _p(yq), _p(yk), _p(yv),
+            Nq if yq_stride is None else yq_stride, Nkv if ykv_stride is None else ykv_stride, K, Nq, Nkv,
+            batch), "fused_qkv_matvec_q4k_batched")
+
+    def matvec_q4k(self, x, W, y, K, N, batch=1) -> None:
+        """MetalCompute::matvec_q4k (metal_compute.h:73-79): y = W x on Q4_K weights."""
+        if batch == 1:
+            check(self.lib.granite_hip_matvec_q4k(_p(x), _p(W), _p(y), K, N), "matvec_q4k")
+        else:
+            check(self.lib.granite_hip_matvec_q4k_batched(_p(x), K, _p(W), _p(y), N, K, N, batch),
+                  "matvec_q4k_batched")
+
     def build_tree_mask(self, parent_indices, mask_words, num_nodes) -> None:
         check(self.lib.granite_hip_build_tree_mask(_p(parent_indices), _p(mask_words), num_nodes),
               "build_tree_mask")

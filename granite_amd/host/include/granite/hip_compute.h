@@ -86,6 +86,21 @@ class HipCompute {
     // The rotation (from cos/sin tables or evaluated) fused with the K/V append.
     Result<void> rope_append(const granite_hip_rope_args& args);
 
+    // MetalCompute::fused_qkv_matvec_q4k (include/granite/metal_compute.h:683-694): the three
+    // attention projections of one token from Q4_K weights [N, K/256] in one launch; x [K],
+    // yq [Nq], yk and yv [Nkv] float.
+    Result<void> fused_qkv_matvec_q4k(HipBuffer* x, HipBuffer* Wq, HipBuffer* Wk, HipBuffer* Wv,
+                                      HipBuffer* yq, HipBuffer* yk, HipBuffer* yv, uint32_t K,
+                                      uint32_t Nq, uint32_t Nkv);
+    // The same for the tokens of a batched decode step: x [batch, K], yq [batch, Nq], yk and
+    // yv [batch, Nkv], the layouts PagedDecodeBatch::run_layer takes.
+    Result<void> fused_qkv_matvec_q4k_batched(HipBuffer* x, HipBuffer* Wq, HipBuffer* Wk,
+                                              HipBuffer* Wv, HipBuffer* yq, HipBuffer* yk,
+                                              HipBuffer* yv, uint32_t K, uint32_t Nq, uint32_t Nkv,
+                                              uint32_t batch);
+    // MetalCompute::matvec_q4k (metal_compute.h:73-79): y [N] = W x, the output projection.
+    Result<void> matvec_q4k(HipBuffer* x, HipBuffer* W, HipBuffer* y, uint32_t K, uint32_t N);
+
     // General entry points (strided Q/out, fp16 or fp32, paged or contiguous
     // keys, causal / tree masks, optional log-sum-exp).
     Result<void> attention(const granite_hip_attention_args& args);

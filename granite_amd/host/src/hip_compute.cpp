@@ -169,6 +169,22 @@ Result<void> HipCompute::decode_attention(const granite_hip_decode_args& args) {
     return HIP_CALL(granite_hip_decode_attention(&args));
 }
 
+Result<void> HipCompute::fused_qkv_matvec_q4k(HipBuffer* x, HipBuffer* Wq, HipBuffer* Wk,
+                                              HipBuffer* Wv, HipBuffer* yq, HipBuffer* yk,
+                                              HipBuffer* yv, uint32_t K, uint32_t Nq, uint32_t Nkv) {
+    return HIP_CALL(granite_hip_fused_qkv_matvec_q4k(x, Wq, Wk, Wv, yq, yk, yv, K, Nq, Nkv));
+}
+Result<void> HipCompute::fused_qkv_matvec_q4k_batched(HipBuffer* x, HipBuffer* Wq, HipBuffer* Wk,
+                                                      HipBuffer* Wv, HipBuffer* yq, HipBuffer* yk,
+                                                      HipBuffer* yv, uint32_t K, uint32_t Nq,
+                                                      uint32_t Nkv, uint32_t batch) {
+    return HIP_CALL(granite_hip_fused_qkv_matvec_q4k_batched(x, K, Wq, Wk, Wv, yq, yk, yv, Nq, Nkv, K,
+                                                             Nq, Nkv, batch));
+}
+Result<void> HipCompute::matvec_q4k(HipBuffer* x, HipBuffer* W, HipBuffer* y, uint32_t K, uint32_t N) {
+    return HIP_CALL(granite_hip_matvec_q4k(x, W, y, K, N));
+}
+
 size_t HipCompute::workspace_bytes() const { return granite_hip_workspace_bytes(); }
 Result<void> HipCompute::reserve_workspace(size_t bytes) {
     return HIP_CALL(granite_hip_reserve_workspace(bytes));

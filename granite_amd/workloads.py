@@ -279,3 +279,81 @@ def make_chunked_prefill(seed=SEED_BASE + 4, prefix_len=32768, chunk=512, num_he
     return ChunkedPrefillCase(q, k_new, v_new, k_pool, v_pool, table, prefix_len, chunk,
                               block_size, num_heads, num_kv_heads, head_dim,
                               float(1.0 / np.sqrt(np.float32(head_dim))))
+
+
+# ---- Q4_K weights (the projections either side of attention) --------------------
+
+QK_K = 256             # weights per super-block
+Q4K_BLOCK_BYTES = 144  # half d, half dmin, 12 bytes of 6-bit scales / minima, 128 bytes of nibbles
+
+
+def pack_q4k(d: np.ndarray, dmin: np.ndarray, scales: np.ndarray, mins: np.ndarray,
+             q: np.ndarray) -> np.ndarray:
+    """Q4_K super-blocks [nb, 144] uint8 from their fields: d, dmin [nb] half; scales, mins
+    [nb, 8] in 0..63; q [nb, 256] in 0..15.  The 6-bit fields are packed the way ggml's
+    quantiser packs them (sub-blocks 0..3 in the low six bits of bytes 0..7, sub-blocks 4..7
+    split between the nibbles of bytes 8..11 and the top two bits of bytes 0..7); of every
+    64 weights the first 32 take the low nibbles of 32 bytes, the next 32 the high ones."""
+    nb = d.shape[0]
+    out = np.zeros((nb, Q4K_BLOCK_BYTES), np.uint8)
+    out[:, 0:2] = np.ascontiguousarray(d, np.float16).view(np.uint8).reshape(nb, 2)
+    out[:, 2:4] = np.ascontiguousarray(dmin, np.float16).view(np.uint8).reshape(nb, 2)
+    ls, lm = scales.astype(np.uint8), mins.astype(np.uint8)
+    packed = out[:, 4:16]
+    for j in range(8):
+        if j < 4:
+            packed[:, j] |= ls[:, j]
+            packed[:, j + 4] |= lm[:, j]
+        else:
+            packed[:, j + 4] = (ls[:, j] & 0xF) | ((lm[:, j] & 0xF) << 4)
+            packed[:, j - 4] |= (ls[:, j] >> 4) << 6
+            packed[:, j] |= (lm[:, j] >> 4) << 6
+    q = q.astype(np.uint8).reshape(nb, 4, 2, 32)
+    out[:, 16:] = (q[:, :, 0, :] | (q[:, :, 1, :] << 4)).reshape(nb, 128)
+    return out
+
+
+@dataclass
+class QkvProjectionCase:
+    """x [batch, K] float32 and the three Q4_K weight matrices of a fused Q/K/V projection
+    ([N, K/256] super-blocks, row major: weight row n holds the K inputs of output n)."""
+    x: np.ndarray
+    wq: np.ndarray   # [Nq, K/256, 144] uint8
+    wk: np.ndarray   # [Nkv, K/256, 144]
+    wv: np.ndarray
+    K: int
+    Nq: int
+    Nkv: int
+
+    @property
+    def batch(self) -> int:
+        return int(self.x.shape[0])
+
+    def algorithmic_bytes(self) -> int:
+        out = self.batch * (self.Nq + 2 * self.Nkv) * 4
+        return self.wq.nbytes + self.wk.nbytes + self.wv.nbytes + self.x.nbytes + out
+
+    def flops(self) -> int:
+        return 2 * self.batch * self.K * (self.Nq + 2 * self.Nkv)
+
+
+def random_q4k(rng: np.random.Generator, rows: int, K: int) -> np.ndarray:
+    """Random Q4_K rows whose dequantised weights look like a trained matrix's (|w| of a
+    few hundredths): every field of the format is drawn, so all code paths of the
+    dequantisation are exercised."""
+    nb = rows * (K // QK_K)
+    d = (rng.uniform(0.5, 1.5, nb) * 4e-4).astype(np.float16)
+    dmin = (rng.uniform(0.5, 1.5, nb) * 4e-4).astype(np.float16)
+    scales = rng.integers(0, 64, (nb, 8))
+    mins = rng.integers(0, 64, (nb, 8))
+    q = rng.integers(0, 16, (nb, QK_K))
+    return pack_q4k(d, dmin, scales, mins, q).reshape(rows, K // QK_K, Q4K_BLOCK_BYTES)
+
+
+def make_qkv_projection(seed=SEED_BASE + 6, K=4096, num_heads=32, num_kv_heads=8, head_dim=128,
+                        batch=1) -> QkvProjectionCase:
+    rng = np.random.default_rng(seed)
+    nq, nkv = num_heads * head_dim, num_kv_heads * head_dim
+    x = _normal(rng, (batch, K))
+    return QkvProjectionCase(x, random_q4k(rng, nq, K), random_q4k(rng, nkv, K), random_q4k(rng, nkv, K),
+                             K, nq, nkv)

@@ -122,7 +122,7 @@ int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
  * While enabled every launch is bracketed by two events on the launch stream.
  * Names: "kv_append", "kv_gather", "decode_stream" or "decode_splitk",
  * "decode_merge", "attention_tiles", "attention_merge", "tree_mask", "rope_append",
- * "mfma_rate".  granite_hip_kernel_timing_names() writes the
+ * "matvec_q4k", "mfma_rate".  granite_hip_kernel_timing_names() writes the
  * names seen so far, comma separated. */
 int granite_hip_enable_kernel_timing(int enable);
 int granite_hip_reset_kernel_timing(void);
@@ -392,6 +392,38 @@ typedef struct granite_hip_rope_args {
 } granite_hip_rope_args;
 
 int granite_hip_rope_append(const granite_hip_rope_args *args);
+
+/* ---- projections either side of attention, on Q4_K weights ----------------- *
+ * A weight matrix is [N, K / 256] Q4_K super-blocks of 144 bytes, row n holding
+ * the K inputs of output n (half d, half dmin, 12 bytes of 6-bit scales and
+ * minima, 128 bytes of 4-bit values; a weight is d * scale * q - dmin * min,
+ * src/model/gguf.cpp:952-1020).  K is a multiple of 256; x, the weights and
+ * the strides are 16-byte aligned.  Results are float, accumulated in float
+ * from the 4-bit values as the reference's GPU kernels do (no weight is ever
+ * rounded to half, which is what separates them from its CPU path). */
+
+/* MetalCompute::fused_qkv_matvec_q4k (include/granite/metal_compute.h:683-694;
+ * kernel metal_shaders_quant.h:167-295; call sites transformer.mm:2966, 4752):
+ * yq[Nq] = Wq x, yk[Nkv] = Wk x, yv[Nkv] = Wv x for one token, one launch. */
+int granite_hip_fused_qkv_matvec_q4k(const void *x, const void *wq, const void *wk,
+                                     const void *wv, void *yq, void *yk, void *yv, uint32_t K,
+                                     uint32_t Nq, uint32_t Nkv);
+
+/* The same for `batch` tokens (a batched decode step): x [batch, K] with rows
+ * x_stride floats apart, yq [batch, Nq] rows yq_stride apart, yk and yv
+ * [batch, Nkv] rows ykv_stride apart -- the layouts granite_hip_rope_append
+ * takes as q, k and v.  The weights are streamed once per four tokens. */
+int granite_hip_fused_qkv_matvec_q4k_batched(const void *x, int64_t x_stride, const void *wq,
+                                             const void *wk, const void *wv, void *yq, void *yk,
+                                             void *yv, int64_t yq_stride, int64_t ykv_stride,
+                                             uint32_t K, uint32_t Nq, uint32_t Nkv,
+                                             uint32_t batch);
+
+/* MetalCompute::matvec_q4k (metal_compute.h:73-79; kernel metal_shaders_quant.h:59-163):
+ * y[N] = W x, the output projection behind attention (transformer.mm:2650, 2955). */
+int granite_hip_matvec_q4k(const void *x, const void *w, void *y, uint32_t K, uint32_t N);
+int granite_hip_matvec_q4k_batched(const void *x, int64_t x_stride, const void *w, void *y,
+                                   int64_t y_stride, uint32_t K, uint32_t N, uint32_t batch);
 
 /* Measurement aid with no counterpart in the reference: the rate the matrix cores
  * reach when nothing else runs.  Two workgroups of eight waves per compute unit issue

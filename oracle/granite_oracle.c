@@ -26,6 +26,12 @@
  *   go_paged_cache_*           src/llm/paged_kv_cache.cpp:104-187
  *   go_rope_table              src/llm/rope.cpp:5-22
  *   go_rope_apply              src/llm/rope.cpp:24-92
+ *   go_q4k_dequantize          src/model/gguf.cpp:952-1020  (Q4_K super-blocks)
+ *   go_matmul_transb_fp16      src/llm/math_ops.cpp:67-103  (portable branch)
+ *   go_matvec_q4k              the projection of MetalCompute::fused_qkv_matvec_q4k
+ *                              (src/backend/metal/kernels/metal_shaders_quant.h:167-295):
+ *                              weights dequantised by the formula above, not rounded
+ *                              to half, dot product in fp32
  *
  * Pinning (what fixes each function besides re-reading it):
  *   conversions     all 65536 halves against the compiler's _Float16, the
@@ -45,6 +51,13 @@
  *                   evaluation of the same fp32 angle, and what a rotation fixes:
  *                   pair norms kept, position 0 is the identity, two rotations
  *                   compose, a unit vector maps to (cos, sin).
+ *   Q4_K            the sizes the reference's tests hold (tests/test_gguf.cpp:78, 106:
+ *                   256 values and 144 bytes per block), ggml's published packing of
+ *                   the 6-bit scales and minima run backwards (pack, then unpack, all
+ *                   64 x 64 values in all 8 positions), hand-built blocks with closed-form
+ *                   values, and a float64 numpy dequantisation written independently;
+ *                   go_matmul_transb_fp16 against the reference's own math_ops.cpp in
+ *                   oracle/_ref.
  */
 #define _GNU_SOURCE
 #include <math.h>
@@ -753,4 +766,119 @@ int go_rope_apply(float *x, int seq_len, int num_heads, int head_dim, int start_
         }
     }
     return 0;
+}
+
+
+/* ------------------------------------------------------------------------- */
+/* Q4_K weights and the projections either side of attention                 */
+/* ------------------------------------------------------------------------- */
+
+/* A Q4_K super-block holds 256 weights in 144 bytes: d and dmin (half), 12 bytes of packed
+ * 6-bit scales and minima for 8 sub-blocks of 32, 128 bytes of 4-bit values
+ * (src/model/gguf.cpp:952-960). */
+#define GO_QK_K 256
+#define GO_Q4K_BLOCK_BYTES 144
+
+/* gguf.cpp:963-971 (ggml's get_scale_min_k4): scale and minimum of sub-block j (0..7). */
+void go_q4k_scale_min(int j, const uint8_t *q, uint8_t *sc, uint8_t *m)
+{
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* gguf.cpp:973-1016: weights of `numel` values (whole super-blocks).  out_f32 receives
+ * d * sc * q - dmin * m as the reference forms it in float; out_f16 what the reference
+ * stores, that value through its truncating fp32_to_fp16.  Either may be NULL. */
+void go_q4k_dequantize(const uint8_t *blocks, size_t numel, float *out_f32, uint16_t *out_f16)
+{
+    size_t num_blocks = (numel + GO_QK_K - 1) / GO_QK_K;
+    const uint8_t *src = blocks;
+    for (size_t b = 0; b < num_blocks; b++) {
+        uint16_t d_bits, dmin_bits;
+        memcpy(&d_bits, src, 2);
+        memcpy(&dmin_bits, src + 2, 2);
+        float d = go_fp16_to_fp32(d_bits);
+        float dmin = go_fp16_to_fp32(dmin_bits);
+        const uint8_t *scales = src + 4;
+        const uint8_t *qs = src + 16;
+        int is = 0;
+        for (int j = 0; j < GO_QK_K; j += 64) {
+            uint8_t sc, m;
+            go_q4k_scale_min(is, scales, &sc, &m);
+            float d1 = d * (float)sc, m1 = dmin * (float)m;
+            go_q4k_scale_min(is + 1, scales, &sc, &m);
+            float d2 = d * (float)sc, m2 = dmin * (float)m;
+            for (int l = 0; l < 32; l++) {
+                size_t idx = b * GO_QK_K + j + l;
+                if (idx >= numel) break;
+                float val = d1 * (float)(qs[l] & 0xF) - m1;
+                if (out_f32) out_f32[idx] = val;
+                if (out_f16) out_f16[idx] = go_fp32_to_fp16(val);
+            }
+            for (int l = 0; l < 32; l++) {
+                size_t idx = b * GO_QK_K + j + 32 + l;
+                if (idx >= numel) break;
+                float val = d2 * (float)(qs[l] >> 4) - m2;
+                if (out_f32) out_f32[idx] = val;
+                if (out_f16) out_f16[idx] = go_fp32_to_fp16(val);
+            }
+            qs += 32;
+            is += 2;
+        }
+        src += GO_Q4K_BLOCK_BYTES;
+    }
+}
+
+/* math_ops.cpp:67-103, the branch without Accelerate: B [N, K] half widened to float,
+ * C[m][n] = sum_k A[m][k] * B[n][k], summed in float in the order of k.  This is how the
+ * reference's CPU attention projects Q, K and V (transformer.mm:1623-1634) from weights
+ * that were dequantised to half when the model was loaded. */
+void go_matmul_transb_fp16(const float *A, const uint16_t *B_fp16, float *C, int M, int N, int K)
+{
+    float *B = (float *)malloc((size_t)N * K * sizeof(float));
+    go_fp16_to_fp32_array(B_fp16, B, (size_t)N * K);
+    for (int m = 0; m < M; m++)
+        for (int n = 0; n < N; n++) {
+            float sum = 0;
+            for (int k = 0; k < K; k++) sum += A[(size_t)m * K + k] * B[(size_t)n * K + k];
+            C[(size_t)m * N + n] = sum;
+        }
+    free(B);
+}
+
+struct go_matvec_job {
+    const float *x;
+    const uint8_t *W;
+    float *y;
+    int K, N, batch;
+};
+
+static void go_matvec_q4k_row(size_t n, void *arg)
+{
+    const struct go_matvec_job *job = (const struct go_matvec_job *)arg;
+    const int K = job->K;
+    float *w = (float *)malloc((size_t)K * sizeof(float));
+    go_q4k_dequantize(job->W + n * (size_t)(K / GO_QK_K) * GO_Q4K_BLOCK_BYTES, (size_t)K, w, NULL);
+    for (int b = 0; b < job->batch; b++) {
+        const float *x = job->x + (size_t)b * K;
+        float sum = 0;
+        for (int k = 0; k < K; k++) sum += x[k] * w[k];
+        job->y[(size_t)b * job->N + n] = sum;
+    }
+    free(w);
+}
+
+/* y[b][n] = sum_k x[b][k] * w[n][k] with W [N, K/256] Q4_K super-blocks, the weights in
+ * float exactly as the dequantisation formula gives them (the GPU path multiplies the
+ * 4-bit values directly, metal_shaders_quant.h:244-280; it never rounds a weight to
+ * half).  Rows are spread over threads as the reference spreads work (parallel_for). */
+void go_matvec_q4k(const float *x, const uint8_t *W, float *y, int K, int N, int batch)
+{
+    struct go_matvec_job job = {x, W, y, K, N, batch};
+    go_parallel_for((size_t)N, (size_t)go_get_num_threads(), go_matvec_q4k_row, &job);
 }

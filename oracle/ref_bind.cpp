@@ -37,4 +37,9 @@ size_t ref_parallel_for_count(size_t n, size_t num_threads, uint8_t* visited) {
     return calls.load();
 }
 
+// The reference's own projection routine (portable branch of matmul_transb).
+void ref_matmul_transb_fp16(const float* A, const uint16_t* B_fp16, float* C, int M, int N, int K) {
+    granite::matmul_transb_fp16(A, B_fp16, C, M, N, K);
+}
+
 }  // extern "C"

@@ -60,6 +60,10 @@ class Oracle:
         L.go_rope_table.argtypes = [_f32p, _f32p, _int, _int, _flt]
         L.go_rope_apply.argtypes = [_f32p, _int, _int, _int, _int, _f32p, _f32p, _int]
         L.go_rope_apply.restype = _int
+        L.go_q4k_scale_min.argtypes = [_int, _u8p, _u8p, _u8p]
+        L.go_q4k_dequantize.argtypes = [_u8p, C.c_size_t, _vp, _vp]
+        L.go_matmul_transb_fp16.argtypes = [_f32p, _u16p, _f32p, _int, _int, _int]
+        L.go_matvec_q4k.argtypes = [_f32p, _u8p, _f32p, _int, _int, _int]
         L.go_block_manager_new.argtypes = [_int, _int]
         L.go_block_manager_delete.argtypes = [_vp]
         L.go_block_manager_allocate.restype = _int
@@ -170,6 +174,35 @@ class Oracle:
             raise ValueError("RoPE position out of range")
         return out
 
+    # ---- Q4_K weights and projections
+    def q4k_dequantize(self, blocks: np.ndarray):
+        """blocks [..., 144] uint8 -> (float32 weights, what the reference stores: half bits)."""
+        blocks = np.ascontiguousarray(blocks, np.uint8)
+        numel = blocks.size // 144 * 256
+        w32, w16 = np.empty(numel, np.float32), np.empty(numel, np.uint16)
+        self.lib.go_q4k_dequantize(blocks.reshape(-1), numel, _opt(w32), _opt(w16))
+        return w32, w16
+
+    def matvec_q4k(self, x: np.ndarray, w_blocks: np.ndarray) -> np.ndarray:
+        """x [batch, K] float32, w_blocks [N, K/256, 144] -> y [batch, N] float32."""
+        x = np.ascontiguousarray(x, np.float32)
+        w = np.ascontiguousarray(w_blocks, np.uint8)
+        batch, K = x.shape
+        N = w.shape[0]
+        y = np.empty((batch, N), np.float32)
+        self.lib.go_matvec_q4k(x, w.reshape(-1), y, K, N, batch)
+        return y
+
+    def matmul_transb_fp16(self, a: np.ndarray, b_half_bits: np.ndarray) -> np.ndarray:
+        """a [M, K] float32, b [N, K] half bits -> a @ b.T (the CPU path's projection)."""
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(b_half_bits, np.uint16)
+        M, K = a.shape
+        N = b.shape[0]
+        c = np.empty((M, N), np.float32)
+        self.lib.go_matmul_transb_fp16(a, b, c, M, N, K)
+        return c
+
     def tree_mask(self, parents) -> np.ndarray:
         parents = np.ascontiguousarray(parents, np.int32)
         n = parents.shape[0]
@@ -228,4 +261,5 @@ def load_ref():
     lib.ref_parallel_for_owner.argtypes = [C.c_size_t, C.c_size_t, _i32p]
     lib.ref_parallel_for_count.restype = C.c_size_t
     lib.ref_parallel_for_count.argtypes = [C.c_size_t, C.c_size_t, _u8p]
+    lib.ref_matmul_transb_fp16.argtypes = [_f32p, _u16p, _f32p, _int, _int, _int]
     return lib

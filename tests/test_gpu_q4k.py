@@ -1,0 +1,106 @@
+"""GPU parity of the projections on Q4_K weights (MetalCompute::fused_qkv_matvec_q4k and
+matvec_q4k, include/granite/metal_compute.h:683-694, 73-79) against the oracle's
+dequantise-and-multiply (src/model/gguf.cpp:952-1020).
+
+Tolerance.  Both sides sum K products in float, in different orders (the kernel also
+applies the minima to sums of inputs, as the reference kernel does), so a result may differ
+from the exact value by a few K * 2^-24 of sum |x_k w_k|; the bound asserted is
+8 * 2^-24 * sqrt(K) * sum |x_k w_k| + 1e-6 against the oracle.  The reference's CPU path
+multiplies by weights it truncated to half at load time; the distance to that path is
+asserted too, at the size of that truncation (2^-10 of sum |x_k w_k|)."""
+import numpy as np
+import pytest
+
+from granite_amd import GraniteHipError, _capi
+from granite_amd import workloads as W
+from gpu_util import dev, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _abs_dot(oracle, x, blocks):
+    w32, _ = oracle.q4k_dequantize(blocks)
+    w = np.abs(w32.astype(np.float64)).reshape(blocks.shape[0], -1)
+    return np.abs(x).astype(np.float64) @ w.T
+
+
+def _check(oracle, got, x, blocks, what):
+    want = oracle.matvec_q4k(x, blocks)
+    mag = _abs_dot(oracle, x, blocks)
+    K = x.shape[1]
+    bound = 8 * 2.0 ** -24 * np.sqrt(K) * mag + 1e-6
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.isfinite(got).all() and np.all(err <= bound), \
+        f"{what}: max err {err.max():.3e}, worst ratio to bound {np.max(err / bound):.2f}"
+    # and the CPU path: the same product with the weights it stored as half
+    _, w16 = oracle.q4k_dequantize(blocks)
+    cpu = oracle.matmul_transb_fp16(x, w16.reshape(blocks.shape[0], K))
+    assert np.all(np.abs(got - cpu) <= 2.0 ** -10 * mag + 2 * bound), f"{what}: off the CPU path"
+    return float(err.max())
+
+
+@pytest.mark.parametrize("K,heads,kv_heads,head_dim,batch", [(256, 1, 1, 8, 1), (512, 3, 1, 24, 1),
+                                                            (2304, 4, 2, 64, 1), (4096, 32, 8, 128, 1),
+                                                            (1024, 5, 1, 64, 2), (2048, 8, 2, 128, 3),
+                                                            (1024, 4, 4, 32, 4), (768, 2, 1, 40, 7)])
+def test_fused_qkv_matvec_q4k(gpu, oracle, K, heads, kv_heads, head_dim, batch):
+    say(f"fused qkv q4k K={K} heads={heads} kv_heads={kv_heads} head_dim={head_dim} batch={batch}")
+    case = W.make_qkv_projection(seed=K + heads + batch, K=K, num_heads=heads, num_kv_heads=kv_heads,
+                                 head_dim=head_dim, batch=batch)
+    yq = dev(np.full((batch, case.Nq), np.nan, np.float32))
+    yk = dev(np.full((batch, case.Nkv), np.nan, np.float32))
+    yv = dev(np.full((batch, case.Nkv), np.nan, np.float32))
+    gpu.fused_qkv_matvec_q4k(dev(case.x), dev(case.wq), dev(case.wk), dev(case.wv), yq, yk, yv, K, case.Nq,
+                             case.Nkv, batch=batch)
+    gpu.sync()
+    _check(oracle, yq.read(np.float32, (batch, case.Nq)), case.x, case.wq, "yq")
+    _check(oracle, yk.read(np.float32, (batch, case.Nkv)), case.x, case.wk, "yk")
+    _check(oracle, yv.read(np.float32, (batch, case.Nkv)), case.x, case.wv, "yv")
+
+
+def test_matvec_q4k_output_projection(gpu, oracle):
+    """y = Wo x with K = num_heads * head_dim: MetalCompute::matvec_q4k behind attention."""
+    rng = np.random.default_rng(3)
+    K, N = 4096, 1000   # a row count that is no multiple of the rows a workgroup takes
+    x = rng.standard_normal((1, K), dtype=np.float32)
+    w = W.random_q4k(rng, N, K)
+    y = dev(np.full((1, N), np.nan, np.float32))
+    gpu.matvec_q4k(dev(x), dev(w), y, K, N)
+    gpu.sync()
+    _check(oracle, y.read(np.float32, (1, N)), x, w, "y")
+    x5 = rng.standard_normal((5, K), dtype=np.float32)
+    y5 = dev(np.full((5, N), np.nan, np.float32))
+    gpu.matvec_q4k(dev(x5), dev(w), y5, K, N, batch=5)
+    gpu.sync()
+    _check(oracle, y5.read(np.float32, (5, N)), x5, w, "y batch 5")
+
+
+def test_known_blocks(gpu):
+    """Hand-built blocks with closed-form results: d = 1, scales 1, no minimum -> the weights
+    are the nibbles; x = 1 -> y = sum of the nibbles; then the minimum alone."""
+    K = 512
+    q = (np.arange(2 * K) * 7 % 16).reshape(4, 256)          # 2 rows x 2 blocks
+    ones, zeros = np.ones(4, np.float16), np.zeros(4, np.float16)
+    w = W.pack_q4k(ones, zeros, np.ones((4, 8)), np.zeros((4, 8)), q).reshape(2, 2, 144)
+    x = np.ones((1, K), np.float32)
+    y = dev(np.zeros((1, 2), np.float32))
+    gpu.matvec_q4k(dev(x), dev(w), y, K, 2)
+    gpu.sync()
+    assert np.array_equal(y.read(np.float32, (1, 2))[0], q.reshape(2, 512).sum(axis=1).astype(np.float32))
+    mins = np.arange(32).reshape(4, 8) % 64
+    w = W.pack_q4k(zeros, np.full(4, 0.5, np.float16), np.ones((4, 8)), mins, q).reshape(2, 2, 144)
+    gpu.matvec_q4k(dev(x), dev(w), y, K, 2)
+    gpu.sync()
+    want = -(0.5 * 32 * mins.reshape(2, 16).sum(axis=1)).astype(np.float32)
+    assert np.array_equal(y.read(np.float32, (1, 2))[0], want)
+
+
+def test_rejects_bad_arguments(gpu):
+    buf = dev(np.zeros(1 << 14, np.float32))
+    lib = _capi.load()
+    assert lib.granite_hip_matvec_q4k(buf.ptr, buf.ptr, buf.ptr, 300, 4) == _capi.EINVAL   # K % 256
+    assert lib.granite_hip_matvec_q4k(None, buf.ptr, buf.ptr, 256, 4) == _capi.ENULL
+    assert lib.granite_hip_matvec_q4k(buf.ptr, None, buf.ptr, 256, 4) == _capi.ENULL
+    assert lib.granite_hip_matvec_q4k(buf.ptr + 4, buf.ptr, buf.ptr, 256, 4) == _capi.EINVAL  # alignment
+    assert lib.granite_hip_matvec_q4k(buf.ptr, buf.ptr, buf.ptr, 256, 0) == _capi.OK
+    gpu.sync()
