@@ -172,7 +172,13 @@ __device__ __forceinline__ uint32_t row_finish(const AttnParams& p, const RowLoo
 }
 
 template <bool kQF32, bool kOutF32, int kRows>
-__global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams p) {
+#ifndef GHIP_PF_OCC
+#define GHIP_PF_OCC 2
+#endif
+#ifndef GHIP_PF_DEEP
+#define GHIP_PF_DEEP 0
+#endif
+__global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
     uint16_t* const s_k0 = s_mem;
     uint16_t* const s_v0 = s_mem + kKBuffers * kKTileHalves;
@@ -535,9 +541,15 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
         const uint16_t* sv = s_v0 + vbuf * kVTileHalves + 32 * sub_v * kVPitch;
         auto k_operand = [&](int s8) -> uint4v {
+#ifdef GHIP_PF_NOLDS
+            return uint4v{uint32_t(s8) + lane, lane, 3u, 4u};
+#endif
             return *reinterpret_cast<const uint4v*>(krow + 16 * s8);
         };
         auto v_operand = [&](int i) -> uint4v {  // step i: head-dim block i & 3, key half i >> 2
+#ifdef GHIP_PF_NOLDS
+            return uint4v{uint32_t(i) + lane, lane, 5u, 6u};
+#endif
             const uint16_t* vp = sv + vt_off[i & 3] + 16 * (i >> 2) * kVPitch;
             const uint2v lo = __builtin_bit_cast(
                 uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -547,10 +559,18 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
                             (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch)));
             return uint4v{lo.x, lo.y, hi.x, hi.y};
         };
+#if GHIP_PF_DEEP
+        // every operand of the phase is requested as early as the registers allow: the eight K
+        // operands at once, the V^T operands one per step of the first half
+        uint4v ka[8], va[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) ka[i] = k_operand(i);
+#else
         constexpr int kRing = 3;
         uint4v ring[kRing];
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(i);
+#endif
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         float psum = 0.0f;
         float pe[16];
@@ -558,6 +578,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
         float tn = __builtin_fmaf(s_in[0], p.scale_log2, -m_ref);
         // the vector work of step e (0..15); element e - 1 is finished here, in pairs
         auto softmax_step = [&](int e) {
+#ifdef GHIP_PF_NOSOFTMAX
+            if (e >= 0) return;
+#endif
             pe[e] = fast_exp2(tn);
             if (e < 15) tn = __builtin_fmaf(s_in[e + 1], p.scale_log2, -m_ref);
             if (e > 0) psum += pe[e - 1];
@@ -565,6 +588,26 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             asm volatile("" : "+v"(pe[e]), "+v"(tn), "+v"(psum));
             if (e > 0 && (e & 1) == 0) asm volatile("" : "+v"(pw[e / 2 - 1]));
         };
+#if GHIP_PF_DEEP
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) {
+            va[s8] = v_operand(s8);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ka[s8]), bq[s8], c, 0, 0, 0);
+            if constexpr (kQF32)
+                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ka[s8]), bq_lo[s8], c, 0, 0, 0);
+            softmax_step(s8);
+            side(s8);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        apply_mask(ti_q, sub_q, c);  // rare
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(va[i]), p_prev[i >> 2], oacc[i & 3], 0, 0, 0);
+            softmax_step(8 + i);
+            side(8 + i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#else
 #pragma unroll
         for (int s8 = 0; s8 < 8; s8++) {
             if (s8 + kRing - 1 < 8) ring[(s8 + kRing - 1) % kRing] = k_operand(s8 + kRing - 1);
@@ -587,6 +630,7 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             side(8 + i);
             __builtin_amdgcn_sched_barrier(0);
         }
+#endif
         psum += pe[15];
         pw[7] = pack_f16x2(pe[14], pe[15]);
         p_out[0] = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
@@ -676,7 +720,11 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             if (piece == 5) look = tile_lookup(it + 6);
         };
         if (fused) {
+#ifdef GHIP_PF_NOSTAGE
+            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old, [](int) {});
+#else
             fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old, [&](int step) { staging(step - 8); });
+#endif
             fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new, [](int) {});
         } else {
 #pragma unroll
@@ -696,7 +744,9 @@ __global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams
             }
         }
         prev_active = cur.active;
+#ifndef GHIP_PF_NOBARRIER
         __syncthreads();
+#endif
         const uint32_t kfreed = kb_cur;
         kb_cur = kb_next;
         kb_next = kb_store;
