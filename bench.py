@@ -583,18 +583,22 @@ EXTRA_WORKLOADS = {"copy_calibration": bench_copy_calibration, "mfma_calibration
 
 
 def main() -> int:
+    global CLOCK_RAMP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS, *EXTRA_WORKLOADS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
+                    help="untimed work in front of every measurement (0 for counter passes)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); the attention path has no "
               "cross-GPU step (it would shard by KV head or by sequence).", file=sys.stderr)
         return 2
 
+    CLOCK_RAMP_MS = args.ramp_ms
     from granite_amd import get_hip_compute
     gpu = get_hip_compute(0)
     info = gpu.device_info()

@@ -9,7 +9,7 @@
 
 namespace ghip {
 
-constexpr int kHeadDim = 128;  // the attention kernels are specialised for D = 128
+constexpr int kHeadDim = 128;  // the largest head size the attention kernels are instantiated for (64 is the other)
 constexpr int kWave = 64;      // CDNA wavefront
 
 // Process-wide launch context (one in-order stream, one scratch buffer).

@@ -42,8 +42,13 @@
 namespace ghip {
 namespace {
 
-template <bool kQF32, int kRows>
+// kD is the head size: 128, or 64 (the reference's d64 decode kernels,
+// metal_shaders_attention.h:2769-2977, 3202-3422).  At 64 a K row gives two MFMA steps
+// instead of four, and only rows 0..7 of the V^T operand (d = 8 m + t < 64) are real: lanes
+// 8..15 of a group repeat the loads of lanes 0..7 and their output rows are dropped.
+template <bool kQF32, int kRows, int kD>
 __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(DecodeParams p) {
+    constexpr int kKSteps = kD / 32;
     // Workgroups go to the 8 XCDs round-robin by linear id, and only the first
     // n_chunks of every (sequence, head) row of the grid carry work.  Rotating
     // the chunk index per row spreads the live chunks evenly over the XCDs;
@@ -72,19 +77,19 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
     const int32_t* table =
         kRows != kRowsContiguous ? p.tables + size_t(b) * p.max_blocks : nullptr;
     const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride + 8 * g;
-    const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * n;
+    const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * (n & (kD / 8 - 1));
 
     // first tile's rows: issued before anything else so the latency overlaps the Q load
     uint32_t row_cur =
         tile_row<kRows>(p, table, chunk_start + min(wave, n_tiles - 1) * kTile, lane, len);
 
     // ---- Q as MFMA B operand: lane (n, g), step s holds Q[qh][32s + 8g .. +7]
-    half8 bq[4];
-    half8 bq_lo[kQF32 ? 4 : 1];
+    half8 bq[kKSteps];
+    half8 bq_lo[kQF32 ? kKSteps : 1];
     {
-        const size_t off = (size_t(b) * p.num_heads + qh) * kHeadDim + 8 * g;
+        const size_t off = (size_t(b) * p.num_heads + qh) * kD + 8 * g;
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
+        for (int s = 0; s < kKSteps; s++) {
             if constexpr (kQF32) {
                 const float* qp = static_cast<const float*>(p.q) + off + 32 * s;
                 float4v x0 = *reinterpret_cast<const float4v*>(qp);
@@ -123,13 +128,13 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
         const uint32_t row_nxt = tile_row<kRows>(p, table, chunk_start + next * kTile, lane, len);
 
         // ---- K tile: two 16-token sub-tiles, 4 k-steps each
-        half8 ka[2][4];
+        half8 ka[2][kKSteps];
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
             const uint32_t row = lane_read(row_cur, 16 * sub + n);
             const uint16_t* kp = kbase + size_t(row) * p.tok_stride;
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+            for (int s = 0; s < kKSteps; s++)
                 ka[sub][s] = as_half8(*reinterpret_cast<const uint4v*>(kp + 32 * s));
         }
         // ---- V tile: 8 token rows per lane, 16 bytes each
@@ -143,7 +148,7 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
         // ---- S^T = K Q^T
         float4v c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
+        for (int s = 0; s < kKSteps; s++) {
             c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[0][s], bq[s], c0, 0, 0, 0);
             c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[1][s], bq[s], c1, 0, 0, 0);
             if constexpr (kQF32) {
@@ -208,7 +213,7 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
     l_run += wave_shfl_xor(l_run, 32);
 
     // ---- merge the 4 waves through LDS
-    constexpr int kRowPad = kHeadDim + 4;
+    constexpr int kRowPad = kD + 4;
     __shared__ float s_o[kWavesPerWG][16][kRowPad];
     __shared__ float s_m[kWavesPerWG][16];
     __shared__ float s_l[kWavesPerWG][16];
@@ -216,15 +221,17 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
         s_m[wave][n] = m_run;
         s_l[wave][n] = l_run;
     }
+    if (32 * g < uint32_t(kD)) {  // output rows 4 g + r of d-tile t are d = 32 g + 8 r + t
 #pragma unroll
-    for (int t = 0; t < 8; t++)
+        for (int t = 0; t < 8; t++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) s_o[wave][n][32 * g + 8 * r + t] = acc[t][r];
+            for (int r = 0; r < 4; r++) s_o[wave][n][32 * g + 8 * r + t] = acc[t][r];
+    }
     __syncthreads();
 
     const uint32_t rows = min(p.group - qg * 16, 16u);
-    for (uint32_t i = threadIdx.x; i < rows * kHeadDim; i += blockDim.x) {
-        const uint32_t row = i / kHeadDim, d = i % kHeadDim;
+    for (uint32_t i = threadIdx.x; i < rows * kD; i += blockDim.x) {
+        const uint32_t row = i / kD, d = i % kD;
         float mx = s_m[0][row];
 #pragma unroll
         for (int w = 1; w < kWavesPerWG; w++) mx = fmaxf(mx, s_m[w][row]);
@@ -238,12 +245,12 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
         const size_t head = size_t(b) * p.num_heads + kvh * p.group + qg * 16 + row;
         if (p.max_chunks == 1) {
             // the only chunk of its (sequence, head): this is the result, no merge launch
-            p.out[head * kHeadDim + d] = o / l;
+            p.out[head * kD + d] = o / l;
             if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
             continue;
         }
         const size_t slot = head * p.max_chunks + chunk;
-        p.part_o[slot * kHeadDim + d] = o;
+        p.part_o[slot * kD + d] = o;
         if (d == 0) {
             p.part_ml[slot * 2 + 0] = mx;
             p.part_ml[slot * 2 + 1] = l;
@@ -254,7 +261,7 @@ __global__ void __launch_bounds__(kWavesPerWG * kWave, 2) decode_splitk_kernel(D
 // Merges the per-chunk partials of one (sequence, query head):
 //   M = max_c m_c,  L = sum_c l_c 2^(m_c - M),  out = sum_c O_c 2^(m_c - M) / L,
 //   lse = (M + log2 L) ln 2.
-__global__ void __launch_bounds__(kHeadDim) decode_merge_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(kHeadDim) decode_merge_kernel(DecodeParams p) {  // head_dim threads
     const uint32_t qh = blockIdx.x;
     const uint32_t b = blockIdx.y;
     uint32_t len = p.seq_lens ? uint32_t(max(p.seq_lens[b], 0)) : p.max_tokens;
@@ -263,7 +270,8 @@ __global__ void __launch_bounds__(kHeadDim) decode_merge_kernel(DecodeParams p) 
     const uint32_t n_chunks = (len + p.chunk_tokens - 1) / p.chunk_tokens;
     const size_t head = size_t(b) * p.num_heads + qh;
     const float* ml = p.part_ml + head * p.max_chunks * 2;
-    const float* po = p.part_o + head * p.max_chunks * kHeadDim;
+    const uint32_t D = p.head_dim;
+    const float* po = p.part_o + head * p.max_chunks * D;
     const uint32_t d = threadIdx.x;
 
     float mx = kNegBig;
@@ -272,9 +280,9 @@ __global__ void __launch_bounds__(kHeadDim) decode_merge_kernel(DecodeParams p) 
     for (uint32_t c = 0; c < n_chunks; c++) {
         const float f = fast_exp2(ml[2 * c] - mx);
         l += ml[2 * c + 1] * f;
-        o += po[size_t(c) * kHeadDim + d] * f;
+        o += po[size_t(c) * D + d] * f;
     }
-    p.out[head * kHeadDim + d] = o / l;
+    p.out[head * D + d] = o / l;
     if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
 }
 
@@ -306,7 +314,8 @@ static bool use_stream_kernel() {
 
 int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch) {
     if (!a.q || !a.k_cache || !a.v_cache || !a.out) return GRANITE_HIP_ENULL;
-    if (a.head_dim != kHeadDim) return GRANITE_HIP_EUNSUPPORTED;
+    if (a.head_dim != 128 && a.head_dim != 64) return GRANITE_HIP_EUNSUPPORTED;
+    const uint32_t D = a.head_dim;
     if (a.num_heads == 0 || a.num_kv_heads == 0 || a.num_heads % a.num_kv_heads != 0)
         return GRANITE_HIP_EINVAL;
     if (a.q_dtype != GRANITE_HIP_F32 && a.q_dtype != GRANITE_HIP_F16) return GRANITE_HIP_EINVAL;
@@ -322,6 +331,7 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
     p.out = static_cast<float*>(a.out);
     p.lse = a.lse;
     p.batch = a.batch_size;
+    p.head_dim = D;
     p.num_heads = a.num_heads;
     p.num_kv_heads = a.num_kv_heads;
     p.group = a.num_heads / a.num_kv_heads;
@@ -331,8 +341,8 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
         p.block_size = a.block_size;
         p.max_blocks = a.max_blocks_per_seq;
         p.bs_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
-        p.tok_stride = int64_t(a.num_kv_heads) * kHeadDim;
-        p.head_stride = kHeadDim;
+        p.tok_stride = int64_t(a.num_kv_heads) * D;
+        p.head_stride = D;
         const uint64_t mt = uint64_t(a.block_size) * a.max_blocks_per_seq;
         if (mt >= (1ull << 31)) return GRANITE_HIP_EINVAL;
         p.max_tokens = static_cast<uint32_t>(mt);
@@ -341,8 +351,8 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
         p.block_size = 1;
         p.max_blocks = 0;
         p.bs_shift = 0;
-        p.tok_stride = kHeadDim;
-        p.head_stride = int64_t(a.max_seq) * kHeadDim;
+        p.tok_stride = D;
+        p.head_stride = int64_t(a.max_seq) * D;
         p.max_tokens = a.max_seq;
     }
     if (!a.seq_lens) {
@@ -375,12 +385,12 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
     int rc = GRANITE_HIP_OK;
     if (p.max_chunks > 1) {
         const size_t slots = size_t(p.batch) * p.num_heads * p.max_chunks;
-        const size_t need = slots * (kHeadDim + 2) * sizeof(float);
+        const size_t need = slots * (D + 2) * sizeof(float);
         void* ws = nullptr;
         rc = take_scratch(scratch, need, &ws);
         if (rc != GRANITE_HIP_OK || scratch.query) return rc;
         p.part_o = static_cast<float*>(ws);
-        p.part_ml = p.part_o + slots * kHeadDim;
+        p.part_ml = p.part_o + slots * D;
     } else if (scratch.query) {
         return GRANITE_HIP_OK;  // one chunk per sequence: the kernel writes the result itself
     }
@@ -390,9 +400,11 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
     hipStream_t st = ctx().stream;
     {
         KernelTimerScope timer("decode_splitk");
-#define GHIP_DECODE_CASE(QF32, ROWS)                                   \
-    if (qf32 == QF32 && rows == ROWS)                                  \
-        decode_splitk_kernel<QF32, ROWS><<<grid, block, 0, st>>>(p);
+#define GHIP_DECODE_CASE(QF32, ROWS)                                        \
+    if (qf32 == QF32 && rows == ROWS) {                                     \
+        if (D == 128) decode_splitk_kernel<QF32, ROWS, 128><<<grid, block, 0, st>>>(p); \
+        else decode_splitk_kernel<QF32, ROWS, 64><<<grid, block, 0, st>>>(p);           \
+    }
         GHIP_DECODE_CASE(true, kRowsContiguous)
         GHIP_DECODE_CASE(true, kRowsPagedPow2)
         GHIP_DECODE_CASE(true, kRowsPagedAny)
@@ -405,7 +417,7 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
     if (rc != GRANITE_HIP_OK || p.max_chunks == 1) return rc;
     {
         KernelTimerScope timer("decode_merge");
-        decode_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(kHeadDim), 0, st>>>(p);
+        decode_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(D), 0, st>>>(p);
     }
     return launch_status();
 }

@@ -24,6 +24,7 @@ struct DecodeParams {
     float* out;
     float* lse;
     uint32_t batch, num_heads, num_kv_heads, group, q_groups;
+    uint32_t head_dim;  // 128 or 64; the kernels are instantiated per head size
     uint32_t block_size, max_blocks;
     int bs_shift;  // log2(block_size) or -1
     int64_t tok_stride, head_stride;

@@ -94,13 +94,17 @@ __device__ __forceinline__ uint32_t list_first_head(const DecodeParams& p, uint3
     return (v0 / p.q_groups) * p.group + (v0 % p.q_groups) * 16;
 }
 
+template <int kD>
 struct TileRegs {
-    half8 ka[2][4];
+    half8 ka[2][kD / 32];
     uint4v vr[8];
 };
 
-template <bool kQF32, int kRows, bool kPair>
+// kD: head size, 128 or 64 (at 64 lanes 8..15 of a group repeat the V loads of lanes 0..7
+// and the output rows they stand for are dropped, as in the chunk kernel).
+template <bool kQF32, int kRows, bool kPair, int kD>
 __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(DecodeParams p) {
+    constexpr int kKSteps = kD / 32;
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15;
@@ -196,16 +200,16 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
     auto head_of = [&](const Cursor& c, uint32_t side) -> uint32_t {
         return kPair ? c.vh * kPairHeads + 2 * wave + side : c.vh;
     };
-    auto issue = [&](TileRegs& r, uint32_t rows, uint32_t vh) {
+    auto issue = [&](TileRegs<kD>& r, uint32_t rows, uint32_t vh) {
         const uint32_t kvh = vh / p.q_groups;
         const uint16_t* kbase = p.k + size_t(kvh) * p.head_stride + 8 * g;
-        const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * n;
+        const uint16_t* vbase = p.v + size_t(kvh) * p.head_stride + 8 * (n & (kD / 8 - 1));
 #pragma unroll
         for (int sub = 0; sub < 2; sub++) {
             const uint32_t row = lane_read(rows, 16 * sub + n);
             const uint16_t* kp = kbase + size_t(row) * p.tok_stride;
 #pragma unroll
-            for (int s = 0; s < 4; s++)
+            for (int s = 0; s < kKSteps; s++)
                 r.ka[sub][s] = as_half8(*reinterpret_cast<const uint4v*>(kp + 32 * s));
         }
 #pragma unroll
@@ -221,8 +225,8 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
     // Running state of one (sequence, virtual head): Q as B operands (with fp32 Q, an fp16
     // head and an fp16 remainder), the maximum, the sum and O.
     struct HeadState {
-        half8 bq[4];
-        half8 bq_lo[kQF32 ? 4 : 1];
+        half8 bq[kKSteps];
+        half8 bq_lo[kQF32 ? kKSteps : 1];
         float m_run, l_run;
         float4v acc[8];
     };
@@ -237,9 +241,9 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
         const uint32_t q_in_group = qg * 16 + n;
         const bool q_valid = q_in_group < p.group;
         const uint32_t qh = kvh * p.group + (q_valid ? q_in_group : 0);
-        const size_t off = (size_t(b) * p.num_heads + qh) * kHeadDim + 8 * g;
+        const size_t off = (size_t(b) * p.num_heads + qh) * kD + 8 * g;
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
+        for (int s = 0; s < kKSteps; s++) {
             if constexpr (kQF32) {
                 const float* qp = static_cast<const float*>(p.q) + off + 32 * s;
                 float4v x0 = *reinterpret_cast<const float4v*>(qp);
@@ -264,11 +268,11 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
         }
     };
 
-    auto compute = [&](const TileRegs& r, const Cursor& c, HeadState& h) {
+    auto compute = [&](const TileRegs<kD>& r, const Cursor& c, HeadState& h) {
         const uint32_t tok0 = c.t * kTile;
         float4v c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
+        for (int s = 0; s < kKSteps; s++) {
             c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[0][s], h.bq[s], c0, 0, 0, 0);
             c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(r.ka[1][s], h.bq[s], c1, 0, 0, 0);
             if constexpr (kQF32) {
@@ -330,13 +334,13 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
         l += wave_shfl_xor(l, 32);
         const uint32_t kvh = vh / p.q_groups, qg = vh % p.q_groups;
         const uint32_t q_in_group = qg * 16 + n;
-        if (q_in_group < p.group) {
+        if (q_in_group < p.group && 32 * g < uint32_t(kD)) {  // (lanes whose rows d = 32 g + .. exist)
             // piece slot = worker + segment; inside it, the query head counted from the
             // first one of the list head
             const uint32_t piece = worker + c.b * lists + c.vh;
             const uint32_t local = kvh * p.group + q_in_group - list_first_head(p, c.vh, kPair);
             const size_t at = size_t(piece) * p.part_cap + local;
-            float* po = p.part_o + at * kHeadDim + 32 * g;
+            float* po = p.part_o + at * kD + 32 * g;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 float4v w;
@@ -359,7 +363,7 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
     Cursor cc = first;  // tile being computed
     Cursor cl = first;  // tile whose K/V rows are requested next
     Cursor cr = first;  // tile whose block-table rows are requested next
-    TileRegs ra, rb;
+    TileRegs<kD> ra, rb;
 
     if constexpr (kPair) {
         // Buffer A always holds the wave's first head of a tile, buffer B its second; both
@@ -452,7 +456,7 @@ __global__ void __launch_bounds__(kWavesPerWG* kWave, 1) decode_stream_kernel(De
 
 // Merges the partials of one (sequence, query head): the workers that touched
 // its list head are consecutive, first = u_start / per, last = (u_end - 1) / per.
-__global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodeParams p) {  // head_dim threads
     const uint32_t qh = blockIdx.x;
     const uint32_t b = blockIdx.y;
     const uint32_t* prefix = p.plan + kPlanHeader;
@@ -472,7 +476,8 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
     const size_t at0 = size_t(first_worker + b * lists + vh) * p.part_cap +
                        (qh - list_first_head(p, vh, heads_per_list > 1));
     const float* ml = p.part_ml + at0 * 2;
-    const float* po = p.part_o + at0 * kHeadDim;
+    const uint32_t D = p.head_dim;
+    const float* po = p.part_o + at0 * D;
     const size_t step = p.part_cap;  // slots of consecutive pieces are part_cap heads apart
     const uint32_t d = threadIdx.x;
 
@@ -482,9 +487,9 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
     for (uint32_t c = 0; c < n_parts; c++) {
         const float f = fast_exp2(ml[2 * c * step] - mx);
         l += ml[2 * c * step + 1] * f;
-        o += po[c * step * kHeadDim + d] * f;
+        o += po[c * step * D + d] * f;
     }
-    p.out[head * kHeadDim + d] = o / l;
+    p.out[head * D + d] = o / l;
     if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
 }
 
@@ -513,14 +518,14 @@ int launch_decode_stream(DecodeParams p, bool q_f32, int rows, const ScratchSour
     const size_t slots = (size_t(workers) + size_t(p.batch) * lists) * p.part_cap;
     const size_t plan_words = kPlanHeader + size_t(p.batch) + 1;
     const size_t plan_bytes = (plan_words * sizeof(uint32_t) + 255) & ~size_t(255);
-    const size_t need = plan_bytes + slots * (kHeadDim + 2) * sizeof(float);
+    const size_t need = plan_bytes + slots * (p.head_dim + 2) * sizeof(float);
     void* ws_ptr = nullptr;
     int rc = take_scratch(scratch, need, &ws_ptr);
     if (rc != GRANITE_HIP_OK || scratch.query) return rc;
     char* ws = static_cast<char*>(ws_ptr);
     p.plan = reinterpret_cast<uint32_t*>(ws);
     p.part_o = reinterpret_cast<float*>(ws + plan_bytes);
-    p.part_ml = p.part_o + slots * kHeadDim;
+    p.part_ml = p.part_o + slots * p.head_dim;
 
     p.workers = workers;
     p.min_per = min_per;
@@ -530,12 +535,17 @@ int launch_decode_stream(DecodeParams p, bool q_f32, int rows, const ScratchSour
     {
         KernelTimerScope timer("decode_stream");
         dim3 grid(wgs), block(kWavesPerWG * kWave);
-#define GHIP_STREAM_CASE(QF32, ROWS)                                             \
-    if (q_f32 == QF32 && rows == ROWS) {                                         \
-        if (pair)                                                                \
-            decode_stream_kernel<QF32, ROWS, true><<<grid, block, lds_bytes, st>>>(p);  \
-        else                                                                     \
-            decode_stream_kernel<QF32, ROWS, false><<<grid, block, lds_bytes, st>>>(p); \
+        const bool d128 = p.head_dim == 128;
+#define GHIP_STREAM_CASE(QF32, ROWS)                                                       \
+    if (q_f32 == QF32 && rows == ROWS) {                                                   \
+        if (pair && d128)                                                                  \
+            decode_stream_kernel<QF32, ROWS, true, 128><<<grid, block, lds_bytes, st>>>(p);  \
+        else if (pair)                                                                     \
+            decode_stream_kernel<QF32, ROWS, true, 64><<<grid, block, lds_bytes, st>>>(p);   \
+        else if (d128)                                                                     \
+            decode_stream_kernel<QF32, ROWS, false, 128><<<grid, block, lds_bytes, st>>>(p); \
+        else                                                                               \
+            decode_stream_kernel<QF32, ROWS, false, 64><<<grid, block, lds_bytes, st>>>(p);  \
     }
         GHIP_STREAM_CASE(true, kRowsContiguous)
         GHIP_STREAM_CASE(true, kRowsPagedPow2)
@@ -549,7 +559,7 @@ int launch_decode_stream(DecodeParams p, bool q_f32, int rows, const ScratchSour
     if (rc != GRANITE_HIP_OK) return rc;
     {
         KernelTimerScope timer("decode_merge");
-        decode_stream_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(kHeadDim), 0, st>>>(p);
+        decode_stream_merge_kernel<<<dim3(p.num_heads, p.batch), dim3(p.head_dim), 0, st>>>(p);
     }
     return launch_status();
 }

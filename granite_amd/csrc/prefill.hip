@@ -81,14 +81,24 @@ namespace {
 constexpr int kBM = 256;       // query rows per workgroup
 constexpr int kBN = 64;        // keys per tile
 constexpr int kThreads = 512;  // 8 waves, two per SIMD
-constexpr int kKPitch = kHeadDim + 8;  // halves per K row in LDS
-constexpr int kVPitch = kHeadDim;      // halves per V row in LDS (chunks swizzled, no padding)
-constexpr int kKTileHalves = kBN * kKPitch;
-constexpr int kVTileHalves = kBN * kVPitch;
 constexpr int kKBuffers = 3;  // K runs a tile ahead of V and is read across two iterations
 constexpr int kVBuffers = 3;  // V of the previous tile is still read while the next is written
-constexpr size_t kLdsBytes =
-    size_t(kKBuffers * kKTileHalves + kVBuffers * kVTileHalves) * sizeof(uint16_t);
+// What depends on the head size kD (128, or 64: the reference's d64 kernels,
+// metal_shaders_attention.h:1447-1660): tile pitches in LDS, MFMA steps of a score
+// product (16 head-dim elements each) and 32-row blocks of the output.
+template <int kD>
+struct Geometry {
+    static_assert(kD == 64 || kD == 128, "head sizes with kernels: 64 and 128");
+    static constexpr int kKPitch = kD + 8;  // halves per K row in LDS
+    static constexpr int kVPitch = kD;      // halves per V row in LDS (chunks swizzled, no padding)
+    static constexpr int kKTileHalves = kBN * kKPitch;
+    static constexpr int kVTileHalves = kBN * kVPitch;
+    static constexpr size_t kLdsBytes =
+        size_t(kKBuffers * kKTileHalves + kVBuffers * kVTileHalves) * sizeof(uint16_t);
+    static constexpr int kSteps = kD / 16;   // MFMAs of the scores of a sub-tile
+    static constexpr int kBlocks = kD / 32;  // 32-row head-dim blocks of O^T; also 64-byte chunks of a V row
+    static constexpr int kPhase = kSteps + 2 * kBlocks;  // MFMAs of a pipeline phase
+};
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -171,14 +181,11 @@ __device__ __forceinline__ uint32_t row_finish(const AttnParams& p, const RowLoo
     }
 }
 
-template <bool kQF32, bool kOutF32, int kRows>
-#ifndef GHIP_PF_OCC
-#define GHIP_PF_OCC 2
-#endif
-#ifndef GHIP_PF_DEEP
-#define GHIP_PF_DEEP 0
-#endif
-__global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(AttnParams p) {
+template <bool kQF32, bool kOutF32, int kRows, int kD>
+__global__ void __launch_bounds__(kThreads, 2) attention_tiles_kernel(AttnParams p) {
+    using G = Geometry<kD>;
+    constexpr int kKPitch = G::kKPitch, kVPitch = G::kVPitch, kKTileHalves = G::kKTileHalves,
+                  kVTileHalves = G::kVTileHalves, kSteps = G::kSteps, kBlocks = G::kBlocks, kPhase = G::kPhase;
     extern __shared__ __attribute__((aligned(16))) uint16_t s_mem[];
     uint16_t* const s_k0 = s_mem;
     uint16_t* const s_v0 = s_mem + kKBuffers * kKTileHalves;
@@ -244,16 +251,16 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
 
     const uint16_t* ka_base = p.k + size_t(kvh) * p.a_head_stride;
     const uint16_t* va_base = p.v + size_t(kvh) * p.a_head_stride;
-    const uint16_t* kb_base = p.k_extra ? p.k_extra + size_t(kvh) * len_b * kHeadDim : nullptr;
-    const uint16_t* vb_base = p.v_extra ? p.v_extra + size_t(kvh) * len_b * kHeadDim : nullptr;
+    const uint16_t* kb_base = p.k_extra ? p.k_extra + size_t(kvh) * len_b * kD : nullptr;
+    const uint16_t* vb_base = p.v_extra ? p.v_extra + size_t(kvh) * len_b * kD : nullptr;
 
     // ---- Q^T as B operand: lane (n, g), step s holds Q[q][16 s + 8 g .. +7]
-    half8 bq[8];
-    half8 bq_lo[kQF32 ? 8 : 1];
+    half8 bq[kSteps];
+    half8 bq_lo[kQF32 ? kSteps : 1];
     {
         const int64_t qoff = int64_t(q_ld) * p.q_tok_stride + int64_t(head) * p.q_head_stride;
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
+        for (int s = 0; s < kSteps; s++) {
             if constexpr (kQF32) {
                 const float* qp = static_cast<const float*>(p.q) + qoff + 16 * s + 8 * g;
                 float4v x0 = *reinterpret_cast<const float4v*>(qp);
@@ -303,22 +310,25 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
 
     float m_ref = kNegBig;  // reference maximum (log2 domain) the probabilities are relative to
     float l_run = 0.0f;     // lane-partial sum (the two k-groups are added at the end)
-    float16v oacc[4];
+    float16v oacc[kBlocks];
 #pragma unroll
-    for (int t = 0; t < 4; t++)
+    for (int t = 0; t < kBlocks; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[t][r] = 0.0f;
 
     // ---- tile staging: this thread moves two 16-byte pieces of key ld_r, columns ld_c and
-    // ld_c + 8 of the 256-byte row, of K and of V: one row lookup and one address per
-    // thread and tile, and every load instruction still covers whole 128-byte lines.
+    // ld_c + 8 of the 256-byte row, of K and of V (head size 64: one piece of the 128-byte
+    // row): one row lookup and one address per thread and tile, and every load instruction
+    // still covers whole 128-byte lines.
     static_assert(kThreads == 8 * kBN, "two 16-byte pieces of one row per thread");
+    constexpr bool kTwoPieces = kD == 128;
     const uint32_t ld_c = tid & 7;   // 16-byte column of the first piece
     const uint32_t ld_r = tid >> 3;  // key inside the tile, 0 .. 63
-    // V: chunk (col >> 2) of row `key` is stored at chunk (col >> 2) ^ (key & 3); the second
-    // piece is two chunks further
-    const uint32_t v_st = ld_r * kVPitch + ((((ld_c >> 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
-    const uint32_t v_st2 = ld_r * kVPitch + (((((ld_c >> 2) + 2) ^ (ld_r & 3)) << 5) | ((ld_c & 3) << 3));
+    // V: the 64-byte chunk (col >> 2) of row `key` is stored at chunk (col >> 2) ^ (key mod
+    // chunks per row); the second piece is two chunks further
+    constexpr uint32_t kSwz = kBlocks - 1;
+    const uint32_t v_st = ld_r * kVPitch + ((((ld_c >> 2) ^ (ld_r & kSwz)) << 5) | ((ld_c & 3) << 3));
+    const uint32_t v_st2 = ld_r * kVPitch + (((((ld_c >> 2) + 2) ^ (ld_r & kSwz)) << 5) | ((ld_c & 3) << 3));
     const uint32_t k_st = ld_r * kKPitch + 8 * ld_c;
 
     // two register sets: the loads of an iteration are stored two iterations later
@@ -342,11 +352,11 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
         it = min(it, n_tiles - 1);
         const bool seg_b = it >= tiles_a;
         const uint16_t* kb = (seg_b ? kb_base : ka_base) + 8 * ld_c;
-        const int64_t stride = seg_b ? int64_t(kHeadDim) : p.a_tok_stride;
+        const int64_t stride = seg_b ? int64_t(kD) : p.a_tok_stride;
         const int64_t off = int64_t(row) * stride;
         const uint4v* src = reinterpret_cast<const uint4v*>(kb + off);
         kreg[0] = src[0];
-        kreg[1] = src[8];
+        if constexpr (kTwoPieces) kreg[1] = src[8];
         return off;
     };
     auto load_v = [&](uint32_t it, int64_t off, uint4v (&vreg)[2]) {
@@ -355,39 +365,40 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
         const uint16_t* vb = (seg_b ? vb_base : va_base) + 8 * ld_c;
         const uint4v* src = reinterpret_cast<const uint4v*>(vb + off);
         vreg[0] = src[0];
-        vreg[1] = src[8];
+        if constexpr (kTwoPieces) vreg[1] = src[8];
     };
     auto store_k_piece = [&](uint32_t buf, const uint4v (&kreg)[2], int piece) {
+        if (piece && !kTwoPieces) return;
         uint4v* dst = reinterpret_cast<uint4v*>(s_k0 + buf * kKTileHalves + k_st);
         dst[8 * piece] = kreg[piece];
     };
     auto store_v_piece = [&](uint32_t buf, const uint4v (&vreg)[2], int piece) {
+        if (piece && !kTwoPieces) return;
         uint16_t* sv = s_v0 + buf * kVTileHalves;
         *reinterpret_cast<uint4v*>(sv + (piece ? v_st2 : v_st)) = vreg[piece];
     };
     auto store_k = [&](uint32_t buf, const uint4v (&kreg)[2]) {
-        uint4v* dst = reinterpret_cast<uint4v*>(s_k0 + buf * kKTileHalves + k_st);
-        dst[0] = kreg[0];
-        dst[8] = kreg[1];
+        store_k_piece(buf, kreg, 0);
+        store_k_piece(buf, kreg, 1);
     };
     auto store_v = [&](uint32_t buf, const uint4v (&vreg)[2]) {
-        uint16_t* sv = s_v0 + buf * kVTileHalves;
-        *reinterpret_cast<uint4v*>(sv + v_st) = vreg[0];
-        *reinterpret_cast<uint4v*>(sv + v_st2) = vreg[1];
+        store_v_piece(buf, vreg, 0);
+        store_v_piece(buf, vreg, 1);
     };
 
     // ---- V^T operand reads.  16-lane group q = lane / 16, lane i = 4k + r inside it:
     // the lane points at key 4 g + k (plus the step's first key), head-dim elements
     // 32 t + 16 (q & 1) + 8 (r & 1) + 4 (r >> 1) .. + 3, and receives, as row n of the A
     // operand, one head-dim element of four consecutive keys.
-    uint32_t vt_off[4];  // halves, per head-dim block t
+    uint32_t vt_off[kBlocks];  // halves, per head-dim block t
     {
         const uint32_t q4 = lane >> 4, i16 = lane & 15;
         const uint32_t k4 = i16 >> 2, r4 = i16 & 3;
         const uint32_t key = 4 * g + k4;
         const uint32_t in_chunk = 16 * (q4 & 1) + 8 * (r4 & 1) + 4 * (r4 >> 1);
 #pragma unroll
-        for (uint32_t t = 0; t < 4; t++) vt_off[t] = key * kVPitch + (((t ^ k4) << 5) | in_chunk);
+        for (uint32_t t = 0; t < uint32_t(kBlocks); t++)
+            vt_off[t] = key * kVPitch + (((t ^ (k4 & kSwz)) << 5) | in_chunk);
     }
 
     // ---- per-tile pieces
@@ -412,7 +423,7 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
         const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub + n) * kKPitch + 8 * g;
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int s8 = 0; s8 < 8; s8++) {
+        for (int s8 = 0; s8 < kSteps; s8++) {
             const half8 a = as_half8(*reinterpret_cast<const uint4v*>(krow + 16 * s8));
             c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[s8], c, 0, 0, 0);
             if constexpr (kQF32) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[s8], c, 0, 0, 0);
@@ -465,7 +476,7 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
         m_ref = m_new;
         l_run *= alpha;
 #pragma unroll
-        for (int t = 0; t < 4; t++)
+        for (int t = 0; t < kBlocks; t++)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[t][r] *= alpha;
     };
@@ -502,7 +513,7 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
     auto accumulate = [&](uint32_t vbuf, int sub, const half8 (&bp)[2]) {
         const uint16_t* sv = s_v0 + vbuf * kVTileHalves + 32 * sub * kVPitch;
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < kBlocks; t++) {
 #pragma unroll
             for (int u = 0; u < 2; u++) {
                 // keys 16 u + {0, 8} + 4 g + (0..3) of the sub-tile: k-index 8 g + 4 a' + b
@@ -531,7 +542,7 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
     // transcendentals run beside it, so a few vector instructions between MFMAs are free
     // while the same instructions after a burst of MFMAs are not.  The scheduling barriers
     // and the empty asm statements keep the compiler from regrouping or sinking the slices.
-    // side(step) is called after the vector work of every step (0..15) for work of the
+    // side(step) is called after the vector work of every step (0 .. kPhase - 1) for work of the
     // caller's that should issue in the shadow of the MFMAs (the tile staging).
     // Operands are fetched from LDS two steps ahead.  Step e scales element e + 1, takes the
     // exponential of element e and sums / packs element e - 1.
@@ -541,16 +552,10 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
         const uint16_t* krow = s_k0 + kbuf * kKTileHalves + (32 * sub_q + n) * kKPitch + 8 * g;
         const uint16_t* sv = s_v0 + vbuf * kVTileHalves + 32 * sub_v * kVPitch;
         auto k_operand = [&](int s8) -> uint4v {
-#ifdef GHIP_PF_NOLDS
-            return uint4v{uint32_t(s8) + lane, lane, 3u, 4u};
-#endif
             return *reinterpret_cast<const uint4v*>(krow + 16 * s8);
         };
-        auto v_operand = [&](int i) -> uint4v {  // step i: head-dim block i & 3, key half i >> 2
-#ifdef GHIP_PF_NOLDS
-            return uint4v{uint32_t(i) + lane, lane, 5u, 6u};
-#endif
-            const uint16_t* vp = sv + vt_off[i & 3] + 16 * (i >> 2) * kVPitch;
+        auto v_operand = [&](int i) -> uint4v {  // step i: head-dim block i % kBlocks, key half i / kBlocks
+            const uint16_t* vp = sv + vt_off[i % kBlocks] + 16 * (i / kBlocks) * kVPitch;
             const uint2v lo = __builtin_bit_cast(
                 uint2v, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                             (short4v __attribute__((address_space(3)))*)(vp)));
@@ -559,18 +564,10 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
                             (short4v __attribute__((address_space(3)))*)(vp + 8 * kVPitch)));
             return uint4v{lo.x, lo.y, hi.x, hi.y};
         };
-#if GHIP_PF_DEEP
-        // every operand of the phase is requested as early as the registers allow: the eight K
-        // operands at once, the V^T operands one per step of the first half
-        uint4v ka[8], va[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) ka[i] = k_operand(i);
-#else
         constexpr int kRing = 3;
         uint4v ring[kRing];
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(i);
-#endif
         float16v c = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         float psum = 0.0f;
         float pe[16];
@@ -578,9 +575,6 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
         float tn = __builtin_fmaf(s_in[0], p.scale_log2, -m_ref);
         // the vector work of step e (0..15); element e - 1 is finished here, in pairs
         auto softmax_step = [&](int e) {
-#ifdef GHIP_PF_NOSOFTMAX
-            if (e >= 0) return;
-#endif
             pe[e] = fast_exp2(tn);
             if (e < 15) tn = __builtin_fmaf(s_in[e + 1], p.scale_log2, -m_ref);
             if (e > 0) psum += pe[e - 1];
@@ -588,49 +582,34 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
             asm volatile("" : "+v"(pe[e]), "+v"(tn), "+v"(psum));
             if (e > 0 && (e & 1) == 0) asm volatile("" : "+v"(pw[e / 2 - 1]));
         };
-#if GHIP_PF_DEEP
+        // the 16 elements are spread evenly over the phase's MFMAs (one each at head size
+        // 128, two each at 64)
+        constexpr int kPer = 16 / kPhase;
+        auto vector_work = [&](int step) {
 #pragma unroll
-        for (int s8 = 0; s8 < 8; s8++) {
-            va[s8] = v_operand(s8);
-            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ka[s8]), bq[s8], c, 0, 0, 0);
-            if constexpr (kQF32)
-                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ka[s8]), bq_lo[s8], c, 0, 0, 0);
-            softmax_step(s8);
-            side(s8);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        apply_mask(ti_q, sub_q, c);  // rare
+            for (int j = 0; j < kPer; j++) softmax_step(step * kPer + j);
+            side(step);
+        };
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(va[i]), p_prev[i >> 2], oacc[i & 3], 0, 0, 0);
-            softmax_step(8 + i);
-            side(8 + i);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#else
-#pragma unroll
-        for (int s8 = 0; s8 < 8; s8++) {
-            if (s8 + kRing - 1 < 8) ring[(s8 + kRing - 1) % kRing] = k_operand(s8 + kRing - 1);
+        for (int s8 = 0; s8 < kSteps; s8++) {
+            if (s8 + kRing - 1 < kSteps) ring[(s8 + kRing - 1) % kRing] = k_operand(s8 + kRing - 1);
             c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq[s8], c, 0, 0, 0);
             if constexpr (kQF32)
                 c = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq_lo[s8], c, 0, 0, 0);
-            softmax_step(s8);
-            side(s8);
+            vector_work(s8);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = v_operand(i);
         apply_mask(ti_q, sub_q, c);  // rare
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            if (i + kRing - 1 < 8) ring[(i + kRing - 1) % kRing] = v_operand(i + kRing - 1);
-            oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[i % kRing]),
-                                                                 p_prev[i >> 2], oacc[i & 3], 0, 0, 0);
-            softmax_step(8 + i);
-            side(8 + i);
+        for (int i = 0; i < 2 * kBlocks; i++) {
+            if (i + kRing - 1 < 2 * kBlocks) ring[(i + kRing - 1) % kRing] = v_operand(i + kRing - 1);
+            oacc[i % kBlocks] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                as_half8(ring[i % kRing]), p_prev[i / kBlocks], oacc[i % kBlocks], 0, 0, 0);
+            vector_work(kSteps + i);
             __builtin_amdgcn_sched_barrier(0);
         }
-#endif
         psum += pe[15];
         pw[7] = pack_f16x2(pe[14], pe[15]);
         p_out[0] = as_half8(uint4v{pw[0], pw[1], pw[2], pw[3]});
@@ -720,11 +699,8 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
             if (piece == 5) look = tile_lookup(it + 6);
         };
         if (fused) {
-#ifdef GHIP_PF_NOSTAGE
-            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old, [](int) {});
-#else
-            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old, [&](int step) { staging(step - 8); });
-#endif
+            fused_phase(cur, kb_cur, 1, s1, s0, p_new, vb_prev, 1, p_old,
+                        [&](int step) { staging(step - (kPhase - 8)); });
             fused_phase(nxt, kb_next, 0, s0, s1, p_old, vb_cur, 0, p_new, [](int) {});
         } else {
 #pragma unroll
@@ -744,9 +720,7 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
             }
         }
         prev_active = cur.active;
-#ifndef GHIP_PF_NOBARRIER
         __syncthreads();
-#endif
         const uint32_t kfreed = kb_cur;
         kb_cur = kb_next;
         kb_next = kb_store;
@@ -775,9 +749,9 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
     if (p.n_splits > 1) {
         // partial result of this key range: O unnormalised, (m_ref, l) beside it
         const size_t row = (size_t(split) * p.num_heads + head) * p.seq_q + q_row;
-        float* po = p.part_o + row * kHeadDim;
+        float* po = p.part_o + row * kD;
 #pragma unroll
-        for (int t = 0; t < 4; t++)
+        for (int t = 0; t < kBlocks; t++)
 #pragma unroll
             for (int ah = 0; ah < 2; ah++) {
                 float x[8];
@@ -799,7 +773,7 @@ __global__ void __launch_bounds__(kThreads, GHIP_PF_OCC) attention_tiles_kernel(
     // head-dim element 32 t + 16 (a >> 1) + 8 g + 4 (a & 1) + b: 8 consecutive elements
     // per (t, a >> 1).
 #pragma unroll
-    for (int t = 0; t < 4; t++)
+    for (int t = 0; t < kBlocks; t++)
 #pragma unroll
         for (int ah = 0; ah < 2; ah++) {
             float x[8];
@@ -839,13 +813,14 @@ __global__ void tree_mask_kernel(const int32_t* parents, uint32_t* mask, uint32_
     }
 }
 
-// Combines the split-K partials of 16 query rows of one head: one thread per
-// (row, 8 consecutive head-dim elements).
-template <bool kOutF32>
+// Combines the split-K partials of 16 (head size 64: 32) query rows of one head: one
+// thread per (row, 8 consecutive head-dim elements).
+template <bool kOutF32, int kD>
 __global__ void __launch_bounds__(256) attention_merge_kernel(AttnParams p, uint32_t n_splits) {
+    constexpr uint32_t kLanesPerRow = kD / 8, kRowsPerGroup = 256 / kLanesPerRow;
     const uint32_t head = blockIdx.y;
-    const uint32_t q_row = blockIdx.x * 16 + (threadIdx.x >> 4);
-    const uint32_t dc = threadIdx.x & 15;
+    const uint32_t q_row = blockIdx.x * kRowsPerGroup + threadIdx.x / kLanesPerRow;
+    const uint32_t dc = threadIdx.x % kLanesPerRow;
     if (q_row >= p.seq_q) return;
     float mx = kNegBig;
     for (uint32_t s = 0; s < n_splits; s++) {
@@ -858,7 +833,7 @@ __global__ void __launch_bounds__(256) attention_merge_kernel(AttnParams p, uint
         const size_t row = (size_t(s) * p.num_heads + head) * p.seq_q + q_row;
         const float f = fast_exp2(p.part_ml[row * 2] - mx);
         l += p.part_ml[row * 2 + 1] * f;
-        const float* po = p.part_o + row * kHeadDim + 8 * dc;
+        const float* po = p.part_o + row * kD + 8 * dc;
         const float4v a = *reinterpret_cast<const float4v*>(po);
         const float4v b = *reinterpret_cast<const float4v*>(po + 4);
         o[0] += a.x * f; o[1] += a.y * f; o[2] += a.z * f; o[3] += a.w * f;
@@ -885,10 +860,11 @@ __global__ void __launch_bounds__(256) attention_merge_kernel(AttnParams p, uint
         p.lse[size_t(head) * p.seq_q + q_row] = (mx + __builtin_amdgcn_logf(l)) * kLn2;
 }
 
-template <bool kQF32, bool kOutF32, int kRows>
+template <bool kQF32, bool kOutF32, int kRows, int kD>
 int launch_tiles(const AttnParams& p, dim3 grid) {
-    auto kernel = attention_tiles_kernel<kQF32, kOutF32, kRows>;
-    static bool configured = false;  // the two LDS buffers exceed the 64 KiB default limit
+    auto kernel = attention_tiles_kernel<kQF32, kOutF32, kRows, kD>;
+    constexpr size_t kLdsBytes = Geometry<kD>::kLdsBytes;
+    static bool configured = false;  // the tile buffers exceed the 64 KiB default limit
     if (!configured) {
         GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -899,11 +875,19 @@ int launch_tiles(const AttnParams& p, dim3 grid) {
     return launch_status();
 }
 
-template <bool kQF32, bool kOutF32>
+template <bool kQF32, bool kOutF32, int kD>
 int launch_tiles_rows(const AttnParams& p, dim3 grid, int rows) {
-    if (rows == kRowsContiguous) return launch_tiles<kQF32, kOutF32, kRowsContiguous>(p, grid);
-    if (rows == kRowsPagedPow2) return launch_tiles<kQF32, kOutF32, kRowsPagedPow2>(p, grid);
-    return launch_tiles<kQF32, kOutF32, kRowsPagedAny>(p, grid);
+    if (rows == kRowsContiguous) return launch_tiles<kQF32, kOutF32, kRowsContiguous, kD>(p, grid);
+    if (rows == kRowsPagedPow2) return launch_tiles<kQF32, kOutF32, kRowsPagedPow2, kD>(p, grid);
+    return launch_tiles<kQF32, kOutF32, kRowsPagedAny, kD>(p, grid);
+}
+
+template <int kD>
+int launch_tiles_types(const AttnParams& p, dim3 grid, int rows, bool qf32, bool of32) {
+    if (qf32 && of32) return launch_tiles_rows<true, true, kD>(p, grid, rows);
+    if (qf32 && !of32) return launch_tiles_rows<true, false, kD>(p, grid, rows);
+    if (!qf32 && of32) return launch_tiles_rows<false, true, kD>(p, grid, rows);
+    return launch_tiles_rows<false, false, kD>(p, grid, rows);
 }
 
 }  // namespace
@@ -922,7 +906,8 @@ int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_
 
 int launch_attention(const granite_hip_attention_args& a, const ScratchSource& scratch) {
     if (!a.q || !a.out) return GRANITE_HIP_ENULL;
-    if (a.head_dim != kHeadDim) return GRANITE_HIP_EUNSUPPORTED;
+    if (a.head_dim != 128 && a.head_dim != 64) return GRANITE_HIP_EUNSUPPORTED;
+    const uint32_t D = a.head_dim;
     if (a.num_heads == 0 || a.num_kv_heads == 0 || a.num_heads % a.num_kv_heads != 0)
         return GRANITE_HIP_EINVAL;
     if ((a.q_dtype != GRANITE_HIP_F32 && a.q_dtype != GRANITE_HIP_F16) ||
@@ -955,11 +940,11 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     p.block_size = a.block_table ? a.block_size : 1;
     p.bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz(p.block_size) : -1;
     if (a.block_table) {
-        p.a_tok_stride = int64_t(a.num_kv_heads) * kHeadDim;
-        p.a_head_stride = kHeadDim;
+        p.a_tok_stride = int64_t(a.num_kv_heads) * D;
+        p.a_head_stride = D;
     } else {
-        p.a_tok_stride = kHeadDim;
-        p.a_head_stride = int64_t(a.max_seq) * kHeadDim;
+        p.a_tok_stride = D;
+        p.a_head_stride = int64_t(a.max_seq) * D;
     }
     p.cache_len = a.cache_len;
     p.k_extra = static_cast<const uint16_t*>(a.k_extra);
@@ -1006,7 +991,7 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     const size_t mask_bytes =
         tree ? (size_t(a.extra_len) * p.mask_words * sizeof(uint32_t) + 255) & ~size_t(255) : 0;
     const size_t rows_total = n_splits > 1 ? size_t(n_splits) * a.num_heads * a.seq_q : 0;
-    const size_t need = mask_bytes + rows_total * (kHeadDim + 2) * sizeof(float);
+    const size_t need = mask_bytes + rows_total * (D + 2) * sizeof(float);
     if (scratch.query) {
         *scratch.query = need;
         return GRANITE_HIP_OK;
@@ -1024,7 +1009,7 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
         }
         if (n_splits > 1) {
             p.part_o = reinterpret_cast<float*>(ws + mask_bytes);
-            p.part_ml = p.part_o + rows_total * kHeadDim;
+            p.part_ml = p.part_o + rows_total * D;
             p.final_out = a.out;
             p.final_tok_stride = a.out_tok_stride;
             p.final_head_stride = a.out_head_stride;
@@ -1040,17 +1025,22 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     int rc;
     {
         KernelTimerScope timer("attention_tiles");
-        if (qf32 && of32) rc = launch_tiles_rows<true, true>(p, grid, rows);
-        else if (qf32 && !of32) rc = launch_tiles_rows<true, false>(p, grid, rows);
-        else if (!qf32 && of32) rc = launch_tiles_rows<false, true>(p, grid, rows);
-        else rc = launch_tiles_rows<false, false>(p, grid, rows);
+        rc = D == 128 ? launch_tiles_types<128>(p, grid, rows, qf32, of32)
+                      : launch_tiles_types<64>(p, grid, rows, qf32, of32);
     }
     if (rc != GRANITE_HIP_OK || n_splits == 1) return rc;
     {
         KernelTimerScope timer("attention_merge");
-        dim3 mgrid((a.seq_q + 15) / 16, a.num_heads);
-        if (of32) attention_merge_kernel<true><<<mgrid, dim3(256), 0, ctx().stream>>>(p, n_splits);
-        else attention_merge_kernel<false><<<mgrid, dim3(256), 0, ctx().stream>>>(p, n_splits);
+        const uint32_t rows_per_group = 256 / (D / 8);
+        dim3 mgrid((a.seq_q + rows_per_group - 1) / rows_per_group, a.num_heads);
+        hipStream_t st = ctx().stream;
+        if (D == 128) {
+            if (of32) attention_merge_kernel<true, 128><<<mgrid, dim3(256), 0, st>>>(p, n_splits);
+            else attention_merge_kernel<false, 128><<<mgrid, dim3(256), 0, st>>>(p, n_splits);
+        } else {
+            if (of32) attention_merge_kernel<true, 64><<<mgrid, dim3(256), 0, st>>>(p, n_splits);
+            else attention_merge_kernel<false, 64><<<mgrid, dim3(256), 0, st>>>(p, n_splits);
+        }
     }
     return launch_status();
 }

@@ -64,8 +64,8 @@ class HipAttentionOp final : public IOperator {
             return Error(ErrorCode::DTypeMismatch, "K and V must be FP16 (the KV cache type)");
         if (!Q.is_contiguous() || !K.is_contiguous() || !V.is_contiguous())
             return Error(ErrorCode::InvalidArgument, "Q, K and V must be contiguous");
-        if (q.dim != 128)
-            return Error(ErrorCode::NotImplemented, "HipAttentionOp has kernels for head_dim 128 only");
+        if (q.dim != 128 && q.dim != 64)
+            return Error(ErrorCode::NotImplemented, "HipAttentionOp has kernels for head_dim 64 and 128");
         return {};
     }
 

@@ -1,0 +1,234 @@
+"""Collects rocprofv3 evidence for the benchmark workloads and writes the short summaries that
+live under profiles/ (one markdown file per workload, plus profiles/traffic.json, which
+bench.py reads for `roofline.traffic`).
+
+    python -m granite_amd.profile_summary collect [workload ...]    # on the GPU box
+    python -m granite_amd.profile_summary summarise [workload ...]  # anywhere, from the raw files
+
+`collect` runs, per workload, one `rocprofv3 --kernel-trace --stats` pass and one `--pmc`
+pass per counter group (every pass is its own process: rocprofv3 does not split counters
+over passes, and a group holds at most 8 SQ counters), always with `python3 bench.py ...`
+as the profiled program.  Raw output goes to gpurun_out/prof/<workload>/; only the summaries
+are meant to be kept.
+"""
+from __future__ import annotations
+
+import collections
+import csv
+import glob
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+RAW = ROOT / "gpurun_out" / "prof"
+PROFILES = ROOT / "profiles"
+
+WORKLOADS = ["paged_decode", "prefill", "chunked_prefill", "tree", "decode_contiguous", "rope_append",
+             "qkv_q4k", "copy_calibration"]
+MFMA_BOUND = {"prefill", "chunked_prefill"}
+DOMINANT = {"paged_decode": "decode_stream_kernel", "prefill": "attention_tiles_kernel",
+            "chunked_prefill": "attention_tiles_kernel", "tree": "attention_tiles_kernel",
+            "decode_contiguous": "decode_splitk_kernel", "rope_append": "rope_append_kernel",
+            "qkv_q4k": "matvec_q4k_kernel", "copy_calibration": "kv_gather_kernel"}
+
+# counter groups: (tag, counters); HBM traffic for every workload, the SQ groups for the
+# MFMA-bound ones (matrix-core utilisation, LDS behaviour, instruction mix, clock)
+TRAFFIC_GROUPS = [("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")]
+SQ_GROUPS = [
+    ("sq1", "SQ_WAVES SQ_WAVE_CYCLES SQ_BUSY_CU_CYCLES SQ_VALU_MFMA_BUSY_CYCLES "
+            "SQ_VALU_MFMA_COEXEC_CYCLES SQ_WAIT_INST_LDS SQ_LDS_BANK_CONFLICT SQ_ACTIVE_INST_VALU"),
+    ("sq2", "SQ_INSTS_VALU SQ_INSTS_MFMA SQ_INSTS_SALU SQ_INSTS_LDS SQ_INSTS_VMEM_RD "
+            "SQ_INSTS_VALU_TRANS_F32 SQ_LDS_IDX_ACTIVE SQ_ACTIVE_INST_LDS"),
+    ("grbm", "GRBM_GUI_ACTIVE"),
+]
+COPY_BYTES = 2 * 65536 * 8 * 128 * 2  # read (and written) by one launch of copy_calibration
+XCDS = 8  # GRBM counters are summed over the part's 8 XCDs
+
+
+def trace_cmd(w: str, out: Path) -> list[str]:
+    return ["rocprofv3", "--kernel-trace", "--stats", "-d", str(out / "trace"), "-o", "t", "--output-format",
+            "csv", "--", "python3", "bench.py", "--workload", w, "--steps", "20", "--warmup", "3", "--no-cpu"]
+
+
+def pmc_cmd(w: str, out: Path, tag: str, counters: str) -> list[str]:
+    return ["rocprofv3", "--pmc", *counters.split(), "-d", str(out / tag), "-o", "p", "--output-format", "csv",
+            "--", "python3", "bench.py", "--workload", w, "--steps", "5", "--warmup", "2", "--no-cpu",
+            "--ramp-ms", "0"]
+
+
+def shown(cmd: list[str]) -> str:
+    """The command as typed from the repository root (raw output under OUT/)."""
+    return " ".join(c.replace(str(RAW) + "/", "OUT/") for c in cmd)
+
+
+def collect(workloads: list[str]) -> int:
+    env = dict(os.environ, TMPDIR="/tmp")
+    for w in workloads:
+        out = RAW / w
+        subprocess.run(["rm", "-rf", str(out)], check=True)
+        out.mkdir(parents=True)
+        groups = TRAFFIC_GROUPS + (SQ_GROUPS if w in MFMA_BOUND else [])
+        cmds = [("trace", trace_cmd(w, out))] + [(tag, pmc_cmd(w, out, tag, c)) for tag, c in groups]
+        for tag, cmd in cmds:
+            print(f"== {w} / {tag}", flush=True)
+            with open(out / f"{tag}.log", "w") as log:
+                # a pass over a short program takes seconds; a hung one is killed, not retried
+                res = subprocess.run(["timeout", "-s", "KILL", "240", *cmd], cwd=ROOT, env=env, stdout=log,
+                                     stderr=subprocess.STDOUT)
+            if res.returncode != 0:
+                print((out / f"{tag}.log").read_text()[-1500:], flush=True)
+                print(f"{w} / {tag} failed with {res.returncode}; stopping", flush=True)
+                return 1
+        for big in glob.glob(str(out / "**" / "*.csv"), recursive=True):
+            if os.path.getsize(big) > 3 << 20:
+                os.remove(big)
+    return 0
+
+
+def short(name: str) -> str:
+    return name.replace("ghip::(anonymous namespace)::", "").replace("ghip::", "").replace("void ", "").split("(")[0]
+
+
+def counters(w: str, tag: str) -> dict:
+    agg = collections.defaultdict(list)
+    for f in glob.glob(str(RAW / w / tag / "**" / "*counter_collection.csv"), recursive=True):
+        for r in csv.DictReader(open(f)):
+            agg[(short(r["Kernel_Name"]).split("<")[0], r["Counter_Name"])].append(float(r["Counter_Value"]))
+    return agg
+
+
+def resources(w: str) -> dict:
+    res = {}
+    for f in glob.glob(str(RAW / w / "trace" / "**" / "*kernel_trace.csv"), recursive=True):
+        for r in csv.DictReader(open(f)):
+            res[short(r["Kernel_Name"])] = (r["VGPR_Count"], r["Accum_VGPR_Count"], r["SGPR_Count"],
+                                            r["LDS_Block_Size"], r["Scratch_Size"], r["Workgroup_Size_X"])
+    return res
+
+
+def clock_ghz(w: str):
+    """GRBM_GUI_ACTIVE cycles over the dispatch's own duration, for the dominant kernel."""
+    ratios = []
+    for f in glob.glob(str(RAW / w / "grbm" / "**" / "*counter_collection.csv"), recursive=True):
+        for r in csv.DictReader(open(f)):
+            if r["Counter_Name"] == "GRBM_GUI_ACTIVE" and short(r["Kernel_Name"]).split("<")[0] == DOMINANT[w]:
+                ns = float(r["End_Timestamp"]) - float(r["Start_Timestamp"])
+                if ns > 0:
+                    ratios.append(float(r["Counter_Value"]) / XCDS / ns)  # the counter sums the 8 XCDs
+    return mean(ratios) if ratios else None
+
+
+def bench_line(w: str) -> dict:
+    for line in open(RAW / w / "trace.log"):
+        if line.startswith("{"):
+            return json.loads(line)
+    raise RuntimeError(f"no bench line in {RAW / w / 'trace.log'}")
+
+
+def mean(v):
+    return sum(v) / len(v)
+
+
+def calibration():
+    f, wr = counters("copy_calibration", "fetch"), counters("copy_calibration", "write")
+    fk = mean([v for (k, c), v in f.items() if "kv_gather" in k][0])
+    wk = mean([v for (k, c), v in wr.items() if "kv_gather" in k][0])
+    return COPY_BYTES / 1024 / fk, COPY_BYTES / 1024 / wk, fk, wk
+
+
+def summarise(workloads: list[str]) -> int:
+    PROFILES.mkdir(exist_ok=True)
+    fetch_kib, write_kib, fetch_raw, write_raw = calibration()
+    traffic_path = PROFILES / "traffic.json"
+    traffic = json.loads(traffic_path.read_text()) if traffic_path.exists() else {}
+    for w in workloads:
+        res = bench_line(w)["workloads"][w]
+        out = RAW / w
+        L = [f"# {w}: rocprofv3 summary ({res['workload']})", "",
+             "Commands (from the repository root on one MI355X, `export TMPDIR=/tmp` first; OUT is any scratch "
+             "folder):", "", "```", shown(trace_cmd(w, out))]
+        groups = TRAFFIC_GROUPS + (SQ_GROUPS if w in MFMA_BOUND else [])
+        L += [shown(pmc_cmd(w, out, tag, c)) for tag, c in groups] + ["```", ""]
+        L += ["## Kernel trace (`*_kernel_stats.csv`: the clock ramp, the warm-up and both timed passes of "
+              "bench.py)", "", "| kernel | calls | avg ns | min ns | max ns | % of GPU time |", "|---|---|---|---|---|---|"]
+        for f in glob.glob(str(out / "trace" / "**" / "*kernel_stats.csv"), recursive=True):
+            for r in csv.DictReader(open(f)):
+                L.append(f"| `{short(r['Name'])[:70]}` | {r['Calls']} | {float(r['AverageNs']):.0f} | {r['MinNs']} | "
+                         f"{r['MaxNs']} | {float(r['Percentage']):.1f} |")
+        L += ["", f"bench.py's own HIP-event timing in the same run, ms per launch: `{json.dumps(res['kernels_ms'])}`; "
+                  f"whole step {res['ms_per_step']} ms."]
+        if "roofline" in res:
+            L += ["", f"Roofline from the event timing: `{json.dumps(res['roofline'])}`"]
+        L += ["", "## Registers, LDS, scratch (kernel trace; LDS is the static part, the K/V tile buffers of "
+              "`attention_tiles_kernel` are 101376 B of dynamic LDS on top)", "",
+              "| kernel | VGPRs | AGPRs | SGPRs | LDS bytes | scratch bytes | workgroup |", "|---|---|---|---|---|---|---|"]
+        for k, v in sorted(resources(w).items()):
+            L.append(f"| `{k[:70]}` | " + " | ".join(v) + " |")
+        L += ["", "## HBM traffic (`FETCH_SIZE`, `WRITE_SIZE`: KiB per dispatch, mean over dispatches)", "",
+              f"Calibration: the identity block-table gather (`--workload copy_calibration`, {COPY_BYTES} B read and "
+              f"as many written per launch) reads FETCH_SIZE = {fetch_raw:.0f} and WRITE_SIZE = {write_raw:.0f}, so one "
+              f"counter unit is {fetch_kib:.3f} KiB of reads and {write_kib:.3f} KiB of writes.", "",
+              "| kernel | FETCH_SIZE | WRITE_SIZE | read bytes (scaled) | written bytes (scaled) |", "|---|---|---|---|---|"]
+        f, wr = counters(w, "fetch"), counters(w, "write")
+        dominant = None
+        for (k, c), v in sorted(f.items()):
+            wv = wr.get((k, "WRITE_SIZE"), [0])
+            rb, wb = mean(v) * fetch_kib * 1024, mean(wv) * write_kib * 1024
+            if k == DOMINANT.get(w):
+                dominant = int(rb + wb)
+            L.append(f"| `{k[:60]}` | {mean(v):.0f} | {mean(wv):.0f} | {rb:.4g} | {wb:.4g} |")
+        if "algorithmic_bytes" in res and dominant is not None:
+            L += ["", f"Algorithmic bytes of the workload: {res['algorithmic_bytes']} per step; traffic of "
+                      f"`{DOMINANT[w]}`: {dominant} B per launch ({dominant / res['algorithmic_bytes']:.3f} x)."]
+            traffic[w] = {"workload": res["workload"], "kernel": DOMINANT[w], "traffic_bytes": dominant,
+                          "summary": f"profiles/{w}.md"}
+        if w in MFMA_BOUND:
+            c = {}
+            for tag, _ in SQ_GROUPS:
+                for (k, name), v in counters(w, tag).items():
+                    if k == DOMINANT[w]:
+                        c[name] = mean(v)
+            L += ["", f"## Matrix-core and LDS counters of `{DOMINANT[w]}` (mean per dispatch)", "",
+                  "| counter | value |", "|---|---|"]
+            L += [f"| {name} | {value:.4g} |" for name, value in sorted(c.items())]
+            if "SQ_BUSY_CU_CYCLES" in c and "SQ_VALU_MFMA_BUSY_CYCLES" in c:
+                busy = c["SQ_VALU_MFMA_BUSY_CYCLES"] / (4 * c["SQ_BUSY_CU_CYCLES"])
+                L += ["", f"Matrix cores busy: SQ_VALU_MFMA_BUSY_CYCLES / (4 SIMDs x SQ_BUSY_CU_CYCLES) = "
+                          f"**{busy:.3f}**"]
+                if "SQ_VALU_MFMA_COEXEC_CYCLES" in c:
+                    L[-1] += (f"; vector ALU running beside them: "
+                              f"{c['SQ_VALU_MFMA_COEXEC_CYCLES'] / (4 * c['SQ_BUSY_CU_CYCLES']):.3f} of the cycles")
+            if "SQ_WAIT_INST_LDS" in c and "SQ_WAVE_CYCLES" in c:
+                L += [f"Waves waiting for LDS: SQ_WAIT_INST_LDS / SQ_WAVE_CYCLES = "
+                      f"{c['SQ_WAIT_INST_LDS'] / c['SQ_WAVE_CYCLES']:.3f}; bank conflicts "
+                      f"{c.get('SQ_LDS_BANK_CONFLICT', 0):.0f} cycles."]
+            if "SQ_WAVES" in c and "SQ_INSTS_MFMA" in c:
+                per = {n: c[n] / c["SQ_WAVES"] for n in c if n.startswith("SQ_INSTS")}
+                L += ["Instructions per wave: " + ", ".join(f"{n[9:]} {v:.0f}" for n, v in sorted(per.items())) + "."]
+            ghz = clock_ghz(w)
+            if ghz:
+                L += [f"Clock under this kernel: GRBM_GUI_ACTIVE / 8 XCDs over the dispatch's own duration (counter "
+                      f"pass: launches serialised, no clock ramp in front) = {ghz:.2f} GHz."]
+        (PROFILES / f"{w}.md").write_text("\n".join(L) + "\n")
+        print(f"wrote profiles/{w}.md", flush=True)
+    traffic_path.write_text(json.dumps(traffic, indent=2) + "\n")
+    return 0
+
+
+def main() -> int:
+    if len(sys.argv) < 2 or sys.argv[1] not in ("collect", "summarise"):
+        print(__doc__)
+        return 2
+    names = sys.argv[2:] or WORKLOADS
+    if sys.argv[1] == "collect":
+        if "copy_calibration" not in names:
+            names = names + ["copy_calibration"]
+        return collect(names)
+    return summarise([n for n in names if n != "copy_calibration"] + (["copy_calibration"] if "copy_calibration" in names else []))
+
+
+if __name__ == "__main__":
+    sys.exit(main())

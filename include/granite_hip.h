@@ -18,10 +18,12 @@
  *     return immediately; results are valid after granite_hip_sync(), exactly
  *     like MetalCompute::sync() (src/backend/metal/metal_compute.mm:150-207);
  *   - "half" means IEEE binary16 stored as uint16_t;
- *   - head_dim must be 128 for the attention entry points
- *     (GRANITE_HIP_EUNSUPPORTED otherwise; the reference rejects head sizes it
- *     has no kernel for, metal_compute.mm:2556-2559); the KV append/gather
- *     entry points accept any head_dim that is a multiple of 8.
+ *   - head_dim must be 128 or 64 for the attention entry points, the two sizes
+ *     the reference has decode and paged kernels for
+ *     (metal_shaders_attention.h:2769-3177, 3202-3847; GRANITE_HIP_EUNSUPPORTED
+ *     otherwise, as the reference rejects other sizes, metal_compute.mm:2556-2559);
+ *     the KV append/gather entry points accept any head_dim that is a multiple
+ *     of 8.
  *
  * Layouts (D = head_dim, G = num_heads / num_kv_heads)
  *   contiguous cache   [num_kv_heads, max_seq, D] half   (src/llm/kv_cache.cpp:20-25)

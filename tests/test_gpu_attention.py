@@ -303,7 +303,7 @@ def test_attention_rejects_bad_arguments(gpu):
     base = dict(q=buf, q_dtype=F32, q_tok_stride=1024, q_head_stride=128, out=buf, out_dtype=F32,
                 out_tok_stride=1024, out_head_stride=128, seq_q=4, num_heads=8, num_kv_heads=2, head_dim=128,
                 scale=0.1, k_cache=buf, v_cache=buf, cache_len=4, max_seq=8, mask_mode=MASK_CAUSAL)
-    for bad, code in ((dict(head_dim=64), _capi.EUNSUPPORTED), (dict(num_kv_heads=3), _capi.EINVAL),
+    for bad, code in ((dict(head_dim=96), _capi.EUNSUPPORTED), (dict(num_kv_heads=3), _capi.EINVAL),
                       (dict(out=None), _capi.ENULL), (dict(max_seq=2), _capi.EINVAL),
                       (dict(mask_mode=9), _capi.EINVAL), (dict(q_tok_stride=1022), _capi.EINVAL),
                       (dict(mask_mode=MASK_TREE), _capi.ENULL), (dict(cache_len=0), _capi.EINVAL),
@@ -311,3 +311,69 @@ def test_attention_rejects_bad_arguments(gpu):
         with pytest.raises(GraniteHipError) as e:
             gpu.attention(**{**base, **bad})
         assert e.value.code == code, bad
+
+
+# ---- head size 64 (the reference's d64 kernels, metal_shaders_attention.h:1447-1660, 2769-2977) ----
+
+@pytest.mark.parametrize("seq,hq,hkv,max_seq", [(1, 4, 4, 8), (65, 8, 2, 100), (128, 4, 2, 128), (300, 16, 4, 300),
+                                                (700, 8, 8, 1024)])
+@pytest.mark.parametrize("q_dtype,out_dtype", [(F16, F16), (F32, F32)])
+def test_causal_prefill_head_dim_64(gpu, oracle, seq, hq, hkv, max_seq, q_dtype, out_dtype):
+    say(f"prefill d64 seq={seq} hq={hq} hkv={hkv} max_seq={max_seq} q={q_dtype} out={out_dtype}")
+    case = W.make_prefill(seed=seq + hq, seq=seq, num_heads=hq, num_kv_heads=hkv, head_dim=64, max_seq=max_seq)
+    q32 = case.q.astype(np.float32)
+    if q_dtype == F32:
+        q32 = q32 + np.random.default_rng(1).standard_normal(q32.shape).astype(np.float32) * 1e-3
+    want, want_lse = oracle.attention_cached(q32[None], case.k_cache, case.v_cache, seq, 0, case.scale)
+    odt = np.float32 if out_dtype == F32 else np.float16
+    out, lse = dev(np.zeros((seq, hq, 64), odt)), dev(np.zeros((hq, seq), np.float32))
+    gpu.attention(q=dev(q32 if q_dtype == F32 else case.q), q_dtype=q_dtype, q_tok_stride=hq * 64, q_head_stride=64,
+                  out=out, out_dtype=out_dtype, out_tok_stride=hq * 64, out_head_stride=64, lse=lse, seq_q=seq,
+                  num_heads=hq, num_kv_heads=hkv, head_dim=64, scale=case.scale, k_cache=dev(case.k_cache),
+                  v_cache=dev(case.v_cache), cache_len=seq, max_seq=max_seq, mask_mode=MASK_CAUSAL, start_pos=0)
+    gpu.sync()
+    assert_close(out.read(odt, (seq, hq, 64)).astype(np.float32), want[0], "out")
+    assert_lse(lse.read(np.float32, (hq, seq)), want_lse[0], "lse")
+
+
+@pytest.mark.parametrize("prefix,chunk,bs,hq,hkv", [(0, 40, 16, 8, 2), (1000, 128, 32, 16, 2), (3000, 96, 16, 8, 2),
+                                                    (511, 300, 12, 4, 1)])
+def test_chunked_prefill_head_dim_64(gpu, oracle, prefix, chunk, bs, hq, hkv):
+    """Paged cache, key splits and the merge kernel at head size 64."""
+    say(f"chunked prefill d64 prefix={prefix} chunk={chunk} bs={bs} hq={hq} hkv={hkv}")
+    case = W.make_chunked_prefill(seed=prefix + chunk, prefix_len=prefix, chunk=chunk, num_heads=hq,
+                                  num_kv_heads=hkv, head_dim=64, block_size=bs, pool_slack=1.5, value_scale=1.0)
+    total = prefix + chunk
+    dk, dv, dt = dev(case.k_pool), dev(case.v_pool), dev(case.block_table)
+    gpu.paged_kv_cache_append_ex(dev(case.k_new), dev(case.v_new), F16, hkv * 64, 64, dk, dv, dt, hkv, 64, prefix,
+                                 chunk, bs)
+    gpu.sync()
+    pool_k, pool_v = dk.read(np.uint16, case.k_pool.shape), dv.read(np.uint16, case.v_pool.shape)
+    want, want_lse = oracle.attention_paged(case.q[None].astype(np.float32), pool_k, pool_v, case.block_table, bs,
+                                            total, prefix, case.scale)
+    out, lse = dev(np.zeros((chunk, hq, 64), np.float16)), dev(np.zeros((hq, chunk), np.float32))
+    gpu.attention(q=dev(case.q), q_dtype=F16, q_tok_stride=hq * 64, q_head_stride=64, out=out, out_dtype=F16,
+                  out_tok_stride=hq * 64, out_head_stride=64, lse=lse, seq_q=chunk, num_heads=hq, num_kv_heads=hkv,
+                  head_dim=64, scale=case.scale, k_cache=dk, v_cache=dv, cache_len=total, block_table=dt,
+                  block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
+    gpu.sync()
+    assert_close(out.read(np.float16, (chunk, hq, 64)).astype(np.float32), want[0], "out")
+    assert_lse(lse.read(np.float32, (hq, chunk)), want_lse[0], "lse")
+
+
+@pytest.mark.parametrize("prefix,n,hq,hkv,bs", [(0, 13, 8, 2, 16), (500, 64, 32, 8, 16), (200, 130, 8, 2, 8)])
+def test_tree_attention_head_dim_64(gpu, oracle, prefix, n, hq, hkv, bs):
+    say(f"tree d64 prefix={prefix} nodes={n} hq={hq} hkv={hkv} bs={bs}")
+    case = W.make_tree(seed=prefix * 5 + n, prefix_len=prefix, num_nodes=n, num_heads=hq, num_kv_heads=hkv,
+                       head_dim=64, block_size=bs, max_children=3, max_depth=12)
+    want, want_lse = _tree_oracle(oracle, case)
+    out, lse = dev(np.zeros((hq, n, 64), np.float32)), dev(np.zeros((hq, n), np.float32))
+    gpu.attention(q=dev(case.q), q_dtype=F32, q_tok_stride=64, q_head_stride=n * 64, out=out, out_dtype=F32,
+                  out_tok_stride=64, out_head_stride=n * 64, lse=lse, seq_q=n, num_heads=hq,
+                  num_kv_heads=hkv, head_dim=64, scale=case.scale, k_cache=dev(case.k_pool), v_cache=dev(case.v_pool),
+                  cache_len=case.prefix_len, block_table=dev(case.block_table) if case.prefix_len else None,
+                  block_size=bs, max_seq=case.prefix_len, k_extra=dev(case.k_tree), v_extra=dev(case.v_tree),
+                  extra_len=n, parents=dev(case.parents), mask_mode=MASK_TREE)
+    gpu.sync()
+    assert_close(out.read(np.float32, (hq, n, 64)), want, "out")
+    assert_lse(lse.read(np.float32, (hq, n)), want_lse, "lse")

@@ -194,10 +194,65 @@ def test_decode_rejects_bad_arguments(gpu):
     buf = dev(np.zeros(4096, np.float32))
     base = dict(q=buf, q_dtype=F32, k_cache=buf, v_cache=buf, out=buf, batch_size=1, num_heads=8,
                 num_kv_heads=2, head_dim=128, scale=0.1, max_seq=16, fixed_seq_len=4)
-    for bad, code in ((dict(head_dim=64), _capi.EUNSUPPORTED), (dict(num_kv_heads=3), _capi.EINVAL),
+    for bad, code in ((dict(head_dim=96), _capi.EUNSUPPORTED), (dict(num_kv_heads=3), _capi.EINVAL),
                       (dict(q=None), _capi.ENULL), (dict(fixed_seq_len=0), _capi.EINVAL),
                       (dict(fixed_seq_len=17), _capi.EINVAL), (dict(chunk_tokens=48), _capi.EINVAL),
                       (dict(q_dtype=7), _capi.EINVAL)):
         with pytest.raises(GraniteHipError) as e:
             gpu.decode_attention(**{**base, **bad})
         assert e.value.code == code, bad
+
+
+# ---- head size 64 (the reference's d64 decode kernels, metal_shaders_attention.h:2769-2977, 3202-3422) ----
+
+def _run_batched_d(gpu, case, q_dtype, D, chunk_tokens=0):
+    B, hq = case.batch, case.num_heads
+    q_host = case.q if q_dtype == F16 else case.q.astype(np.float32)
+    out = dev(np.full((B, hq, D), -7.0, np.float32))
+    lse = dev(np.full((B, hq), -7.0, np.float32))
+    bufs = (dev(q_host), dev(case.k_pool), dev(case.v_pool), dev(case.block_tables), dev(case.seq_lens))
+    gpu.decode_attention(q=bufs[0], q_dtype=q_dtype, k_cache=bufs[1], v_cache=bufs[2], block_tables=bufs[3],
+                         seq_lens=bufs[4], out=out, lse=lse, batch_size=B, num_heads=hq,
+                         num_kv_heads=case.num_kv_heads, head_dim=D, scale=case.scale,
+                         block_size=case.block_size, max_blocks_per_seq=case.max_blocks, chunk_tokens=chunk_tokens)
+    gpu.sync()
+    return out.read(np.float32, (B, hq, D)), lse.read(np.float32, (B, hq))
+
+
+@pytest.mark.parametrize("q_dtype", [F16, F32])
+@pytest.mark.parametrize("hq,hkv,bs,ctx", [(32, 8, 16, 768), (12, 3, 12, 2112), (64, 16, 32, 2112), (40, 2, 16, 600),
+                                           (8, 8, 16, 5000)])
+def test_batched_paged_decode_head_dim_64(gpu, oracle, q_dtype, hq, hkv, bs, ctx):
+    """Both kernels (one workgroup per short context, the persistent one for long ones) and
+    both list shapes of the persistent kernel at head size 64."""
+    lens = np.array([1, 17, 64, 0, 255, 256, 257, ctx, 33, ctx // 2 + 1], np.int32)
+    case = W.make_paged_decode(seed=hq + bs, num_heads=hq, num_kv_heads=hkv, head_dim=64, block_size=bs,
+                               ctx_max=ctx, seq_lens=lens)
+    say(f"batched paged decode d64 hq={hq} hkv={hkv} bs={bs} ctx={ctx} q_dtype={q_dtype}")
+    want, want_lse = oracle.batched_paged_decode(case.q.astype(np.float32), case.k_pool, case.v_pool,
+                                                 case.block_tables, case.seq_lens, bs, case.scale)
+    got, got_lse = _run_batched_d(gpu, case, q_dtype, 64)
+    live = lens > 0
+    assert_close(got[live], want[live], "out")
+    assert_lse(got_lse[live], want_lse[live], "lse")
+    assert np.all(got[~live] == -7.0) and np.all(got_lse[~live] == -7.0)
+    if ctx > 768:   # the chunk kernel with its merge launch as well
+        got, got_lse = _run_batched_d(gpu, case, q_dtype, 64, chunk_tokens=256)
+        assert_close(got[live], want[live], "out (chunk kernel)")
+        assert_lse(got_lse[live], want_lse[live], "lse (chunk kernel)")
+
+
+@pytest.mark.parametrize("seq_kv,max_seq,hq,hkv", [(1, 64, 8, 8), (33, 64, 32, 8), (700, 4096, 40, 2), (3000, 3000, 16, 4)])
+def test_decode_contiguous_head_dim_64(gpu, oracle, seq_kv, max_seq, hq, hkv):
+    say(f"decode contiguous d64 seq_kv={seq_kv} max_seq={max_seq} hq={hq} hkv={hkv}")
+    case = W.make_decode_contiguous(seed=seq_kv, num_heads=hq, num_kv_heads=hkv, head_dim=64, seq_kv=seq_kv,
+                                    max_seq=max_seq)
+    want, want_lse = oracle.attention_cached(case.q[None, None], case.k_cache, case.v_cache, seq_kv, seq_kv - 1,
+                                             case.scale)
+    out, lse = dev(np.zeros((hq, 64), np.float32)), dev(np.zeros(hq, np.float32))
+    gpu.decode_attention(q=dev(case.q), q_dtype=F32, k_cache=dev(case.k_cache), v_cache=dev(case.v_cache),
+                         out=out, lse=lse, batch_size=1, num_heads=hq, num_kv_heads=hkv, head_dim=64,
+                         scale=case.scale, max_seq=max_seq, fixed_seq_len=seq_kv)
+    gpu.sync()
+    assert_close(out.read(np.float32, (hq, 64)), want[0, 0], "out")
+    assert_lse(lse.read(np.float32, (hq,)), want_lse[0, :, 0], "lse")
