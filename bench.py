@@ -408,32 +408,39 @@ def bench_copy_calibration(gpu, steps, warmup, cpu):
 
 
 def bench_mfma_calibration(gpu, steps, warmup, cpu):
-    """The rate the matrix cores reach with nothing else running, on register operands: zeros
-    (the part keeps its peak clock) against normally distributed fp16 values (the power limit
-    holds the clock down), for both MFMA shapes.  The data-like rate is what an MFMA-bound
-    kernel can be compared with beside the published peak.  Not part of `--workload all`."""
-    from granite_amd import DeviceBuffer
+    """What the matrix cores reach on register operands (libgranite_hip_calibration.so, a
+    measurement aid beside the attention library): zeros (the part keeps its peak clock)
+    against normally distributed fp16 values (the power limit holds the clock down), both MFMA
+    shapes, and then with the other instructions an attention inner loop issues per MFMA
+    beside them -- float FMAs, an exponential, a 16-byte LDS operand read -- with one and with
+    two waves per SIMD.  The last line of the mix table (3 FMAs, 1 exponential, 1 LDS read) is
+    the prefill kernel's mix: the rate an MFMA-bound attention kernel can be compared with
+    beside the published peak.  Not part of `--workload all`."""
+    from granite_amd import DeviceBuffer, calibration
     rng = np.random.default_rng(11)
     n = 1 << 20
     data = {"zeros": np.zeros(n, np.float16),
             "normal": (0.05 * rng.standard_normal(n, dtype=np.float32)).astype(np.float16)}
-    rates = {}
-    ms_total = 0.0
-    for kind, host in data.items():
-        buf = DeviceBuffer.from_numpy(host)
-        for shape in (32, 16):
-            flops = [0.0]
+    bufs = {k: DeviceBuffer.from_numpy(v) for k, v in data.items()}
+    iterations = 20000
 
-            def step():
-                flops[0] = gpu.mfma_rate(buf, n, 20000, shape)
+    def rate(kind, shape, waves, mix):
+        best = 0.0
+        for _ in range(max(1, min(steps, 3))):
+            flops, ms = calibration.mfma_rate(bufs[kind], n, iterations, shape=shape, waves_per_simd=waves, mix=mix)
+            best = max(best, flops / (ms * 1e-3) / 1e12)
+        return round(best, 1)
 
-            ms, _, _ = Timer(gpu).run(step, warmup, steps)
-            ms_total += ms
-            rates[f"{kind}_{shape}"] = round(flops[0] / (ms * 1e-3) / 1e12, 1)
-    return {"workload": "mfma_calibration_register_operands_8waves_per_cu", "metric": "mfma_TFLOPs",
-            "unit": "TFLOP/s", "value": rates["normal_32"], "ms_per_step": round(ms_total, 4),
+    rates = {f"{kind}_{shape}": rate(kind, shape, 2, (0, 0, 0)) for kind in data for shape in (32, 16)}
+    mixes = {"mfma_only": (0, 0, 0), "4_fma": (4, 0, 0), "8_fma": (8, 0, 0), "1_exp": (0, 1, 0),
+             "3_fma_1_exp": (3, 1, 0), "1_lds_read": (0, 0, 1), "3_fma_1_exp_1_lds_read": (3, 1, 1)}
+    mix_rates = {name: {f"{w}_wave_per_simd": rate("normal", 32, w, mix) for w in (1, 2)}
+                 for name, mix in mixes.items()}
+    return {"workload": "mfma_calibration_register_operands_one_workgroup_per_cu", "metric": "mfma_TFLOPs",
+            "unit": "TFLOP/s", "value": rates["normal_32"], "ms_per_step": 0.0,
             "rates_TFLOPs": {"zeros_32x32x16": rates["zeros_32"], "zeros_16x16x32": rates["zeros_16"],
                              "normal_32x32x16": rates["normal_32"], "normal_16x16x32": rates["normal_16"]},
+            "instruction_mix_TFLOPs_32x32x16_normal": mix_rates,
             "peak_TFLOPs": 2500.0}
 
 

@@ -178,7 +178,6 @@ SIGNATURES = {
         _int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _u32, _u32, _u32, _u32]),
     "granite_hip_matvec_q4k": (_int, [_vp, _vp, _vp, _u32, _u32]),
     "granite_hip_matvec_q4k_batched": (_int, [_vp, _i64, _vp, _vp, _i64, _u32, _u32, _u32]),
-    "granite_hip_mfma_rate": (_int, [_vp, C.c_uint64, _u32, _int, C.POINTER(C.c_double)]),
     "granite_hip_workspace_bytes": (C.c_size_t, []),
     "granite_hip_reserve_workspace": (_int, [C.c_size_t]),
     "granite_hip_decode_workspace_required": (_int, [C.POINTER(DecodeArgs), C.POINTER(C.c_size_t)]),

@@ -592,14 +592,6 @@ int granite_hip_matvec_q4k(const void* x, const void* w, void* y, uint32_t K, ui
     return granite_hip_matvec_q4k_batched(x, K, w, y, N, K, N, 1);
 }
 
-// ---- measurement aid ----------------------------------------------------------
-
-int granite_hip_mfma_rate(const void* operands_f16, uint64_t n_halves, uint32_t iterations,
-                          int shape, double* flops) {
-    GHIP_REQUIRE_INIT();
-    return ghip::launch_mfma_rate(operands_f16, n_halves, iterations, shape, flops);
-}
-
 // ---- attention ------------------------------------------------------------
 
 int granite_hip_decode_attention(const granite_hip_decode_args* args) {

@@ -109,8 +109,6 @@ int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_
 int launch_rope_append(const granite_hip_rope_args& a);
 int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], void* const y[3],
                       const int64_t y_stride[3], const uint32_t n[3], uint32_t K, uint32_t batch);
-int launch_mfma_rate(const void* operands, uint64_t n_halves, uint32_t iterations, int shape,
-                     double* flops);
 
 // ---- device helpers ------------------------------------------------------
 #if defined(__HIPCC__)

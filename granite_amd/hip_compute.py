@@ -267,13 +267,6 @@ class HipCompute:
         """Grow the library's scratch now, so that later launches needing no more never allocate."""
         check(self.lib.granite_hip_reserve_workspace(nbytes), "reserve_workspace")
 
-    def mfma_rate(self, operands, n_halves: int, iterations: int, shape: int = 32) -> float:
-        """Launches the matrix-core rate kernel on `operands` (fp16 values); returns its flops."""
-        flops = C.c_double(0.0)
-        check(self.lib.granite_hip_mfma_rate(_p(operands), n_halves, iterations, shape, C.byref(flops)),
-              "mfma_rate")
-        return flops.value
-
     def kv_commit_accepted(self, k_tree, v_tree, src_dtype, src_tok_stride, src_head_stride, num_nodes,
                            accepted_nodes, num_accepted, k_cache, v_cache, num_kv_heads, head_dim,
                            start_pos, block_table=None, block_size=0, max_seq_len=0,

@@ -124,7 +124,7 @@ int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
  * While enabled every launch is bracketed by two events on the launch stream.
  * Names: "kv_append", "kv_gather", "decode_stream" or "decode_splitk",
  * "decode_merge", "attention_tiles", "attention_merge", "tree_mask", "rope_append",
- * "matvec_q4k", "mfma_rate".  granite_hip_kernel_timing_names() writes the
+ * "matvec_q4k".  granite_hip_kernel_timing_names() writes the
  * names seen so far, comma separated. */
 int granite_hip_enable_kernel_timing(int enable);
 int granite_hip_reset_kernel_timing(void);
@@ -426,18 +426,6 @@ int granite_hip_fused_qkv_matvec_q4k_batched(const void *x, int64_t x_stride, co
 int granite_hip_matvec_q4k(const void *x, const void *w, void *y, uint32_t K, uint32_t N);
 int granite_hip_matvec_q4k_batched(const void *x, int64_t x_stride, const void *w, void *y,
                                    int64_t y_stride, uint32_t K, uint32_t N, uint32_t batch);
-
-/* Measurement aid with no counterpart in the reference: the rate the matrix cores
- * reach when nothing else runs.  Two workgroups of eight waves per compute unit issue
- * `iterations` passes of 16 v_mfma_f32_32x32x16_f16 (shape 32) or 32
- * v_mfma_f32_16x16x32_f16 (shape 16) on register operands read once from
- * operands_f16 (n_halves halves, a multiple of 8; lane i takes halves [16 i, 16 i + 16)
- * modulo the buffer).  *flops receives the flops of the launch; time it with the events
- * above or the kernel timer (name "mfma_rate").  With zeros the part keeps its peak clock;
- * with data-like operands its power limit holds it lower, and that rate is the one an
- * MFMA-bound kernel can be compared with. */
-int granite_hip_mfma_rate(const void *operands_f16, uint64_t n_halves, uint32_t iterations,
-                          int shape, double *flops);
 
 /* ---- scratch memory ------------------------------------------------------ *
  * Decode and prefill launches that split the keys over several workgroups

@@ -25,6 +25,18 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} declared in granite_hip.h but not exported"
 
 
+def test_calibration_library_exports_its_header():
+    """The measurement aid is a library of its own, beside the attention library."""
+    cal_header = ROOT / "include" / "granite_hip_calibration.h"
+    text = re.sub(r"/\*.*?\*/", "", cal_header.read_text(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(granite_hip_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["granite_hip_cal_mfma_rate"]
+    lib = C.CDLL(str(ROOT / "granite_amd" / "lib" / "libgranite_hip_calibration.so"))
+    for name in names:
+        assert hasattr(lib, name)
+    assert not hasattr(_capi.load(), "granite_hip_cal_mfma_rate")   # and not in the product library
+
+
 def test_binding_table_covers_the_header():
     assert sorted(_capi.SIGNATURES) == declared_symbols()
 

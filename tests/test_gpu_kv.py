@@ -237,17 +237,23 @@ def test_kv_commit_accepted_path(gpu, oracle, paged, src_dtype):
         assert e.value.code == _capi.EOVERFLOW
 
 
-def test_mfma_rate_runs_and_checks_arguments(gpu):
-    """The matrix-core rate kernel (a measurement aid): finishes, reports its flops, and
-    refuses what its launch does not cover."""
-    say("mfma_rate")
-    n = 4096
+def test_calibration_library_runs_and_checks_arguments(gpu):
+    """The matrix-core rate kernel (libgranite_hip_calibration.so, a measurement aid beside
+    the attention library): finishes, reports its flops and its time, and refuses what its
+    launches do not cover."""
+    import ctypes as C
+    from granite_amd import calibration
+    say("calibration library")
+    n = 16384
     buf = dev(np.ones(n, np.float16))
     units = gpu.device_info().compute_units
-    for shape in (32, 16):
-        flops = gpu.mfma_rate(buf, n, 10, shape)
-        gpu.sync()
-        assert flops == 2 * units * 8 * 10 * 16 * 2 * 32 * 32 * 16
-    for n_halves, iterations, shape in ((12, 10, 32), (n, 0, 32), (n, 10, 8)):
-        with pytest.raises(GraniteHipError):
-            gpu.mfma_rate(buf, n_halves, iterations, shape)
+    for shape, waves, mix in ((32, 2, (0, 0, 0)), (16, 2, (0, 0, 0)), (32, 1, (3, 1, 1)), (32, 2, (3, 1, 1))):
+        flops, ms = calibration.mfma_rate(buf, n, 10, shape=shape, waves_per_simd=waves, mix=mix)
+        assert flops == units * 4 * waves * 10 * 16 * 2 * 32 * 32 * 16 and ms > 0
+    for kwargs in (dict(n_halves=12), dict(iterations=0), dict(shape=8), dict(waves_per_simd=3),
+                   dict(mix=(5, 0, 0)), dict(shape=16, mix=(3, 1, 1))):
+        args = dict(n_halves=n, iterations=10, shape=32, waves_per_simd=2, mix=(0, 0, 0))
+        args.update(kwargs)
+        with pytest.raises(RuntimeError):
+            calibration.mfma_rate(buf, args["n_halves"], args["iterations"], shape=args["shape"],
+                                  waves_per_simd=args["waves_per_simd"], mix=args["mix"])
