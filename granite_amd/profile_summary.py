@@ -93,11 +93,34 @@ def short(name: str) -> str:
 
 
 def counters(w: str, tag: str) -> dict:
-    agg = collections.defaultdict(list)
+    """{(kernel, counter): values of the dispatches with the kernel's largest grid} -- a
+    workload that also launches its kernel on a small side shape (rope_append's 512-token
+    chunk) is counted on its main shape only."""
+    rows = collections.defaultdict(list)
     for f in glob.glob(str(RAW / w / tag / "**" / "*counter_collection.csv"), recursive=True):
         for r in csv.DictReader(open(f)):
-            agg[(short(r["Kernel_Name"]).split("<")[0], r["Counter_Name"])].append(float(r["Counter_Value"]))
+            rows[(short(r["Kernel_Name"]).split("<")[0], r["Counter_Name"])].append(
+                (int(r["Grid_Size"]), float(r["Counter_Value"])))
+    agg = {}
+    for key, vals in rows.items():
+        biggest = max(g for g, _ in vals)
+        agg[key] = [v for g, v in vals if g == biggest]
     return agg
+
+
+def main_shape_duration(w: str):
+    """(calls, mean ns) of the dominant kernel's largest-grid dispatches in the kernel trace."""
+    rows = []
+    for f in glob.glob(str(RAW / w / "trace" / "**" / "*kernel_trace.csv"), recursive=True):
+        for r in csv.DictReader(open(f)):
+            if short(r["Kernel_Name"]).split("<")[0] == DOMINANT.get(w):
+                grid = int(r["Grid_Size_X"]) * int(r["Grid_Size_Y"]) * int(r["Grid_Size_Z"])
+                rows.append((grid, float(r["End_Timestamp"]) - float(r["Start_Timestamp"])))
+    if not rows:
+        return None
+    biggest = max(g for g, _ in rows)
+    ns = [d for g, d in rows if g == biggest]
+    return len(ns), mean(ns)
 
 
 def resources(w: str) -> dict:
@@ -158,6 +181,10 @@ def summarise(workloads: list[str]) -> int:
             for r in csv.DictReader(open(f)):
                 L.append(f"| `{short(r['Name'])[:70]}` | {r['Calls']} | {float(r['AverageNs']):.0f} | {r['MinNs']} | "
                          f"{r['MaxNs']} | {float(r['Percentage']):.1f} |")
+        main = main_shape_duration(w)
+        if main:
+            L += ["", f"`{DOMINANT[w]}` on the workload's main shape (largest grid): {main[0]} launches, mean "
+                      f"{main[1]:.0f} ns."]
         L += ["", f"bench.py's own HIP-event timing in the same run, ms per launch: `{json.dumps(res['kernels_ms'])}`; "
                   f"whole step {res['ms_per_step']} ms."]
         if "roofline" in res:
