@@ -481,13 +481,33 @@ __global__ void __launch_bounds__(kHeadDim) decode_stream_merge_kernel(DecodePar
     const size_t step = p.part_cap;  // slots of consecutive pieces are part_cap heads apart
     const uint32_t d = threadIdx.x;
 
-    float mx = kNegBig;
-    for (uint32_t c = 0; c < n_parts; c++) mx = fmaxf(mx, ml[2 * c * step]);
-    float o = 0.0f, l = 0.0f;
-    for (uint32_t c = 0; c < n_parts; c++) {
-        const float f = fast_exp2(ml[2 * c * step] - mx);
-        l += ml[2 * c * step + 1] * f;
-        o += po[c * step * D + d] * f;
+    // One pass, four pieces at a time: the loads of a group do not depend on anything
+    // computed here, so they are all in flight together (two dependent rounds of memory
+    // latency in all: the plan, then the pieces), and the running maximum is folded in
+    // as the groups arrive.
+    float mx = kNegBig, o = 0.0f, l = 0.0f;
+    for (uint32_t c0 = 0; c0 < n_parts; c0 += 4) {
+        float m[4], ls[4], os[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const size_t c = min(c0 + i, n_parts - 1);  // clamped: always a written slot
+            m[i] = ml[2 * c * step];
+            ls[i] = ml[2 * c * step + 1];
+            os[i] = po[c * step * D + d];
+        }
+        float m_new = mx;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) m_new = fmaxf(m_new, c0 + i < n_parts ? m[i] : kNegBig);
+        const float keep = fast_exp2(mx - m_new);
+        o *= keep;
+        l *= keep;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const float f = c0 + i < n_parts ? fast_exp2(m[i] - m_new) : 0.0f;
+            l += ls[i] * f;
+            o += os[i] * f;
+        }
+        mx = m_new;
     }
     p.out[head * D + d] = o / l;
     if (p.lse && d == 0) p.lse[head] = (mx + __builtin_amdgcn_logf(l)) * kLn2;

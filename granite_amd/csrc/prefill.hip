@@ -822,22 +822,39 @@ __global__ void __launch_bounds__(256) attention_merge_kernel(AttnParams p, uint
     const uint32_t q_row = blockIdx.x * kRowsPerGroup + threadIdx.x / kLanesPerRow;
     const uint32_t dc = threadIdx.x % kLanesPerRow;
     if (q_row >= p.seq_q) return;
-    float mx = kNegBig;
-    for (uint32_t s = 0; s < n_splits; s++) {
-        const size_t row = (size_t(s) * p.num_heads + head) * p.seq_q + q_row;
-        mx = fmaxf(mx, p.part_ml[row * 2]);
-    }
-    float l = 0.0f;
+    // One pass, four splits at a time: the loads of a group depend on nothing computed
+    // here, so they are in flight together, and the running maximum is folded in as the
+    // groups arrive.
+    float mx = kNegBig, l = 0.0f;
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (uint32_t s = 0; s < n_splits; s++) {
-        const size_t row = (size_t(s) * p.num_heads + head) * p.seq_q + q_row;
-        const float f = fast_exp2(p.part_ml[row * 2] - mx);
-        l += p.part_ml[row * 2 + 1] * f;
-        const float* po = p.part_o + row * kD + 8 * dc;
-        const float4v a = *reinterpret_cast<const float4v*>(po);
-        const float4v b = *reinterpret_cast<const float4v*>(po + 4);
-        o[0] += a.x * f; o[1] += a.y * f; o[2] += a.z * f; o[3] += a.w * f;
-        o[4] += b.x * f; o[5] += b.y * f; o[6] += b.z * f; o[7] += b.w * f;
+    for (uint32_t s0 = 0; s0 < n_splits; s0 += 4) {
+        float m[4], ls[4];
+        float4v a[4], b[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const uint32_t sp = min(s0 + i, n_splits - 1);  // clamped: always a written row
+            const size_t row = (size_t(sp) * p.num_heads + head) * p.seq_q + q_row;
+            m[i] = p.part_ml[row * 2];
+            ls[i] = p.part_ml[row * 2 + 1];
+            const float* po = p.part_o + row * kD + 8 * dc;
+            a[i] = *reinterpret_cast<const float4v*>(po);
+            b[i] = *reinterpret_cast<const float4v*>(po + 4);
+        }
+        float m_new = mx;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) m_new = fmaxf(m_new, s0 + i < n_splits ? m[i] : kNegBig);
+        const float keep = fast_exp2(mx - m_new);
+        l *= keep;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] *= keep;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const float f = s0 + i < n_splits ? fast_exp2(m[i] - m_new) : 0.0f;
+            l += ls[i] * f;
+            o[0] += a[i].x * f; o[1] += a[i].y * f; o[2] += a[i].z * f; o[3] += a[i].w * f;
+            o[4] += b[i].x * f; o[5] += b[i].y * f; o[6] += b[i].z * f; o[7] += b[i].w * f;
+        }
+        mx = m_new;
     }
     const float inv_l = 1.0f / l;
     const int64_t ooff =
