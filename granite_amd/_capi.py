@@ -156,7 +156,7 @@ SIGNATURES = {
     "granite_hip_paged_kv_cache_append": (
         _int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "granite_hip_paged_kv_cache_append_ex": (
-        _int, [_vp, _vp, _int, _i64, _i64, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _int]),
+        _int, [_vp, _vp, _int, _i64, _i64, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _int, _u32]),
     "granite_hip_paged_kv_gather": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
     "granite_hip_multihead_attention": (
         _int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _f32, _u32]),

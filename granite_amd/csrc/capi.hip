@@ -542,8 +542,12 @@ int granite_hip_paged_kv_cache_append_ex(const void* new_k, const void* new_v, i
                                          void* k_cache, void* v_cache,
                                          const int32_t* block_table, uint32_t num_kv_heads,
                                          uint32_t head_dim, uint32_t start_pos,
-                                         uint32_t new_len, uint32_t block_size, int rounding) {
+                                         uint32_t new_len, uint32_t block_size, int rounding,
+                                         uint32_t max_blocks) {
     GHIP_REQUIRE_INIT();
+    if (max_blocks > 0 && block_size > 0 &&
+        (uint64_t(start_pos) + new_len + block_size - 1) / block_size > max_blocks)
+        return GRANITE_HIP_EOVERFLOW;
     return ghip::launch_kv_append_paged(new_k, new_v, src_dtype, src_tok_stride, src_head_stride,
                                         k_cache, v_cache, block_table, num_kv_heads, head_dim,
                                         start_pos, new_len, block_size, rounding);

@@ -163,11 +163,13 @@ class HipCompute:
 
     def paged_kv_cache_append_ex(self, new_k, new_v, src_dtype, src_tok_stride, src_head_stride,
                                  k_cache, v_cache, block_table, num_kv_heads, head_dim, start_pos,
-                                 new_len, block_size, rounding=ROUND_TRUNCATE) -> None:
+                                 new_len, block_size, rounding=ROUND_TRUNCATE, max_blocks=0) -> None:
+        """max_blocks: entries of block_table (0: not stated); an append that would run past
+        them fails with EOVERFLOW instead of reading beyond the table."""
         check(self.lib.granite_hip_paged_kv_cache_append_ex(
             _p(new_k), _p(new_v), src_dtype, src_tok_stride, src_head_stride, _p(k_cache),
             _p(v_cache), _p(block_table), num_kv_heads, head_dim, start_pos, new_len, block_size,
-            rounding), "paged_kv_cache_append_ex")
+            rounding, max_blocks), "paged_kv_cache_append_ex")
 
     def paged_kv_gather(self, dst_k, dst_v, k_cache, v_cache, block_table, num_kv_heads, head_dim,
                         length, block_size, max_seq_len) -> None:

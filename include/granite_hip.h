@@ -164,13 +164,18 @@ int granite_hip_paged_kv_cache_append(const void *new_k, const void *new_v, void
                                       uint32_t num_kv_heads, uint32_t head_dim,
                                       uint32_t start_pos, uint32_t new_len, uint32_t block_size);
 
-/* General form (strided source, F32 or F16 source, rounding choice). */
+/* General form (strided source, F32 or F16 source, rounding choice).
+ * max_blocks: entries the block table holds; start_pos + new_len tokens must fit
+ * that many blocks or the call fails with GRANITE_HIP_EOVERFLOW before anything is
+ * written.  0: not stated, as in the reference's entry point, which takes no
+ * bound -- a table that is too short is then read past its end. */
 int granite_hip_paged_kv_cache_append_ex(const void *new_k, const void *new_v, int src_dtype,
                                          int64_t src_tok_stride, int64_t src_head_stride,
                                          void *k_cache, void *v_cache,
                                          const int32_t *block_table, uint32_t num_kv_heads,
                                          uint32_t head_dim, uint32_t start_pos,
-                                         uint32_t new_len, uint32_t block_size, int rounding);
+                                         uint32_t new_len, uint32_t block_size, int rounding,
+                                         uint32_t max_blocks);
 
 /* Commit of a speculation tree's accepted path.  After find_accepted_path
  * (src/llm/speculation_tree.cpp:85-143) the runner only truncates the target

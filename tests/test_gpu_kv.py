@@ -131,7 +131,15 @@ def test_paged_append_f16_then_gather_round_trip(gpu, oracle):
     src_v = rng.integers(0, 65536, (total, hkv, d)).astype(np.uint16)
     pk = np.full((pool_blocks * bs, hkv, d), SENT, np.uint16)
     dpk, dpv, dt = dev(pk), dev(pk), dev(table)
-    gpu.paged_kv_cache_append_ex(dev(src_k), dev(src_v), F16, hkv * d, d, dpk, dpv, dt, hkv, d, 0, total, bs)
+    # a table declared one block too short is refused before anything is written
+    with pytest.raises(GraniteHipError) as e:
+        gpu.paged_kv_cache_append_ex(dev(src_k), dev(src_v), F16, hkv * d, d, dpk, dpv, dt, hkv, d, 0, total, bs,
+                                     max_blocks=nblk - 1)
+    assert e.value.code == _capi.EOVERFLOW
+    gpu.sync()
+    assert np.all(dpk.read(np.uint16, pk.shape) == SENT)
+    gpu.paged_kv_cache_append_ex(dev(src_k), dev(src_v), F16, hkv * d, d, dpk, dpv, dt, hkv, d, 0, total, bs,
+                                 max_blocks=nblk)
     want_pool = pk.copy()
     oracle.lib.go_paged_kv_cache_append_f16(want_pool.reshape(-1), src_k.reshape(-1), table, hkv, d, 0,
                                             total, bs, hkv * d, d)
