@@ -19,6 +19,19 @@
 // inputs of a sub-block instead of to every weight, and a nibble is converted with one
 // byte-to-float instruction (the high nibbles stay multiplied by 16, which the scale takes
 // back).  Lanes are combined with shuffles at the end; results are float.
+//
+// A batch of tokens (a batched decode step) goes through the matrix cores instead
+// (matmul_q4k_tokens_kernel): up to 32 tokens per launch are the rows of the MFMA's A operand,
+// 32 weight rows its columns.  What makes that cheap for a 4-bit format: the B operand is not a
+// dequantised weight but the integer scale * q (at most 63 * 15 = 945), written as the raw
+// bits of a half -- a denormal, i.e. exactly scale * q * 2^-24, which the matrix cores keep --
+// so a nibble costs a mask, a byte shuffle and a 24-bit multiply shared between two weights,
+// and nothing is rounded; d * 2^24 is applied once per super-block to the accumulator.  The
+// minima go through one more MFMA per super-block, the integer minima against the sums of
+// the inputs of the sub-blocks.  Inputs are split into a half and a half remainder (two MFMAs
+// per step) so that float inputs lose nothing.  A workgroup stages its 512 input columns in
+// LDS once (both halves, and the sub-block sums) for its 8 waves x 32 weight rows; the chunks
+// of K are combined by a second small kernel.
 #include "common.h"
 
 namespace ghip {
@@ -28,7 +41,7 @@ constexpr uint32_t kQK = 256;          // weights per super-block
 constexpr uint32_t kBlockBytes = 144;  // bytes per super-block
 constexpr int kRowsPerWave = 2;
 constexpr int kWavesPerGroup = 4;
-constexpr int kMaxBatch = 4;  // input vectors one launch multiplies every weight with
+constexpr int kMaxBatch = 2;  // input vectors the vector kernel takes; larger batches go to the matrix cores
 
 struct MatvecParams {
     const float* x;       // [batch, K], rows x_stride floats apart
@@ -199,6 +212,196 @@ __global__ void __launch_bounds__(kWavesPerGroup* kWave) matvec_q4k_kernel(Matve
         }
 }
 
+
+// ---- a batch of tokens on the matrix cores ---------------------------------------------------
+
+constexpr int kTokTile = 32;          // tokens per launch (rows of the A operand)
+constexpr int kTokWaves = 8;          // waves per workgroup, 32 weight rows each
+constexpr int kTokRows = 32 * kTokWaves;
+constexpr int kChunkK = 512;          // input columns a workgroup stages: two super-blocks
+constexpr int kChunkBlocks = kChunkK / int(kQK);
+constexpr int kXPitch = kChunkK + 8;  // halves per token row in LDS (16-byte reads without bank conflicts)
+constexpr int kSubPerChunk = kChunkK / 32;
+constexpr size_t kTokLdsBytes = size_t(2 * kTokTile * kXPitch + 2 * kTokTile * kSubPerChunk) * sizeof(uint16_t);
+
+struct MatmulTokParams {
+    MatvecParams m;   // x, weights and row numbering as for the matvec; m.batch = all tokens
+    float* partial;   // [chunks, token tiles * kTokTile, rows_total]
+    uint32_t chunks;  // ceil(K / kChunkK)
+    uint32_t tokens;  // token tiles * kTokTile
+};
+
+__device__ __forceinline__ uint32_t bytes_to_u16_pair(uint32_t bytes, bool upper) {
+    // bytes [b0 b1 b2 b3] -> b0 | b1 << 16 (or b2 | b3 << 16): one v_perm_b32
+    return __builtin_amdgcn_perm(0u, bytes, upper ? 0x0c030c02u : 0x0c010c00u);
+}
+
+__global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(MatmulTokParams q) {
+    const MatvecParams& p = q.m;
+    extern __shared__ __attribute__((aligned(16))) uint16_t s_tok[];
+    uint16_t* const s_xh = s_tok;                           // [kTokTile][kXPitch] half of x
+    uint16_t* const s_xl = s_xh + kTokTile * kXPitch;       // remainder of x
+    uint16_t* const s_sh = s_xl + kTokTile * kXPitch;       // [kTokTile][kSubPerChunk] sub-block sums
+    uint16_t* const s_sl = s_sh + kTokTile * kSubPerChunk;  // and their remainders
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t n = lane & 31, g = lane >> 5;
+    const uint32_t chunk = blockIdx.y;
+    const uint32_t tok0 = blockIdx.z * kTokTile;          // first token of this workgroup's tile
+    const uint32_t tile_batch = min(p.batch - tok0, uint32_t(kTokTile));
+    const uint32_t k0 = chunk * kChunkK;
+    const uint32_t K = p.blocks_per_row * kQK;
+
+    // ---- this lane's weight row
+    const uint32_t rows_total = p.row_end[2];
+    const uint32_t row = blockIdx.x * kTokRows + wave * 32 + n;
+    const uint32_t rowc = min(row, rows_total - 1);  // clamped: loads stay in bounds, stores are masked
+    const int seg = rowc < p.row_end[0] ? 0 : (rowc < p.row_end[1] ? 1 : 2);
+    const uint32_t local = rowc - (seg == 0 ? 0 : p.row_end[seg - 1]);
+    const uint8_t* wrow = p.w[seg] + size_t(local) * p.blocks_per_row * kBlockBytes;
+
+    // all weight loads of the chunk are requested before anything else, so that their latency
+    // runs beside the staging of the inputs
+    uint4v head[kChunkBlocks], nib[kChunkBlocks][4];
+    bool live_block[kChunkBlocks];
+#pragma unroll
+    for (int sb = 0; sb < kChunkBlocks; sb++) {
+        const uint32_t ib = chunk * kChunkBlocks + sb;
+        live_block[sb] = ib < p.blocks_per_row;
+        const uint8_t* blk = wrow + size_t(min(ib, p.blocks_per_row - 1)) * kBlockBytes;
+        head[sb] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(blk));
+#pragma unroll
+        for (int G = 0; G < 4; G++)
+            nib[sb][G] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(blk + 16 + 32 * G + 16 * g));
+    }
+
+    // ---- stage the chunk's inputs: thread (token, sub-block) converts 32 floats
+    {
+        const uint32_t b = tid / kSubPerChunk, j = tid % kSubPerChunk;
+        const bool live = b < tile_batch && k0 + 32 * j < K;
+        const float* xp = p.x + int64_t(tok0 + min(b, tile_batch - 1)) * p.x_stride + min(k0 + 32 * j, K - 32);
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float4v a = *reinterpret_cast<const float4v*>(xp + 8 * i);
+            const float4v c = *reinterpret_cast<const float4v*>(xp + 8 * i + 4);
+            const float v[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
+            uint32_t hi[4], lo[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float x0 = live ? v[2 * e] : 0.0f, x1 = live ? v[2 * e + 1] : 0.0f;
+                sum += x0 + x1;
+                const _Float16 h0 = static_cast<_Float16>(x0), h1 = static_cast<_Float16>(x1);
+                half2v hh, ll;
+                hh.x = h0;
+                hh.y = h1;
+                ll.x = static_cast<_Float16>(x0 - static_cast<float>(h0));
+                ll.y = static_cast<_Float16>(x1 - static_cast<float>(h1));
+                hi[e] = __builtin_bit_cast(uint32_t, hh);
+                lo[e] = __builtin_bit_cast(uint32_t, ll);
+            }
+            *reinterpret_cast<uint4v*>(s_xh + b * kXPitch + 32 * j + 8 * i) = uint4v{hi[0], hi[1], hi[2], hi[3]};
+            *reinterpret_cast<uint4v*>(s_xl + b * kXPitch + 32 * j + 8 * i) = uint4v{lo[0], lo[1], lo[2], lo[3]};
+        }
+        const _Float16 sh = static_cast<_Float16>(sum);
+        s_sh[b * kSubPerChunk + j] = __builtin_bit_cast(uint16_t, sh);
+        s_sl[b * kSubPerChunk + j] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(sum - static_cast<float>(sh)));
+    }
+    __syncthreads();
+
+    float y[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) y[r] = 0.0f;
+#pragma unroll
+    for (int sb = 0; sb < kChunkBlocks; sb++) {
+        // integer scales and minima of the 8 sub-blocks (gguf.cpp:963-971)
+        uint32_t sc[8], mn[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; j++) {
+            if (j < 4) {
+                sc[j] = scale_byte(head[sb], j) & 63u;
+                mn[j] = scale_byte(head[sb], j + 4) & 63u;
+            } else {
+                sc[j] = (scale_byte(head[sb], j + 4) & 0xFu) | ((scale_byte(head[sb], j - 4) >> 6) << 4);
+                mn[j] = (scale_byte(head[sb], j + 4) >> 4) | ((scale_byte(head[sb], j) >> 6) << 4);
+            }
+        }
+        float16v acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int G = 0; G < 4; G++) {
+            // the lane's 16 bytes of group G: low nibbles are inputs 64 G + 16 g + 0..15 (scale 2 G),
+            // high nibbles the inputs 32 further on (scale 2 G + 1)
+#pragma unroll
+            for (int part = 0; part < 4; part++) {  // 8 inputs each: low 0..7, low 8..15, high 0..7, high 8..15
+                const bool high = part >= 2;
+                const uint32_t w0 = nib[sb][G][2 * (part & 1)], w1 = nib[sb][G][2 * (part & 1) + 1];
+                const uint32_t q0 = (high ? (w0 >> 4) : w0) & 0x0F0F0F0Fu;
+                const uint32_t q1 = (high ? (w1 >> 4) : w1) & 0x0F0F0F0Fu;
+                const uint32_t scale = sc[2 * G + (high ? 1 : 0)];
+                uint4v bw;  // scale * q as raw half bits: scale * q * 2^-24 exactly
+                bw.x = __umul24(bytes_to_u16_pair(q0, false), scale);
+                bw.y = __umul24(bytes_to_u16_pair(q0, true), scale);
+                bw.z = __umul24(bytes_to_u16_pair(q1, false), scale);
+                bw.w = __umul24(bytes_to_u16_pair(q1, true), scale);
+                const uint32_t kk = sb * kQK + 64 * G + (high ? 32 : 0) + 16 * g + 8 * (part & 1);
+                const half8 ah = __builtin_bit_cast(half8, *reinterpret_cast<const uint4v*>(s_xh + n * kXPitch + kk));
+                const half8 al = __builtin_bit_cast(half8, *reinterpret_cast<const uint4v*>(s_xl + n * kXPitch + kk));
+                const half8 bb = __builtin_bit_cast(half8, bw);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bb, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bb, acc, 0, 0, 0);
+            }
+        }
+        // minima: sum_j min_j * (sum of the inputs of sub-block j), j on the contraction axis
+        float16v accm = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        {
+            uint4v bm = {mn[0] | (mn[1] << 16), mn[2] | (mn[3] << 16), mn[4] | (mn[5] << 16), mn[6] | (mn[7] << 16)};
+            uint4v sh = *reinterpret_cast<const uint4v*>(s_sh + n * kSubPerChunk + 8 * sb);
+            uint4v sl = *reinterpret_cast<const uint4v*>(s_sl + n * kSubPerChunk + 8 * sb);
+            if (g == 1) {  // only 8 of the 16 contraction slots are used
+                bm = uint4v{0, 0, 0, 0};
+                sh = uint4v{0, 0, 0, 0};
+                sl = uint4v{0, 0, 0, 0};
+            }
+            accm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, sh), __builtin_bit_cast(half8, bm), accm, 0, 0, 0);
+            accm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, sl), __builtin_bit_cast(half8, bm), accm, 0, 0, 0);
+        }
+        const half2v dd = __builtin_bit_cast(half2v, head[sb].x);
+        const float d = live_block[sb] ? float(dd.x) * 16777216.0f : 0.0f;      // the integers were worth 2^-24
+        const float dmin = live_block[sb] ? float(dd.y) * 16777216.0f : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) y[r] += d * acc[r] - dmin * accm[r];
+    }
+
+    // ---- this chunk's part of y: register r is token 8 (r / 4) + 4 g + r % 4, the lane's column its row
+    if (row < rows_total) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t b = 8 * (r >> 2) + 4 * g + (r & 3);
+            if (b < tile_batch) q.partial[(size_t(chunk) * q.tokens + tok0 + b) * rows_total + row] = y[r];
+        }
+    }
+}
+
+// y[token][row] = sum over the chunks of K; one thread per (row, token)
+__global__ void __launch_bounds__(256) matmul_q4k_tokens_merge_kernel(MatmulTokParams q) {
+    const MatvecParams& p = q.m;
+    const uint32_t rows_total = p.row_end[2];
+    const uint32_t row = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t b = blockIdx.y;
+    if (row >= rows_total) return;
+    float sum = 0.0f;
+    for (uint32_t c0 = 0; c0 < q.chunks; c0 += 8) {  // eight loads in flight, summed in chunk order
+        float part[8];
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++)
+            part[i] = q.partial[(size_t(min(c0 + i, q.chunks - 1)) * q.tokens + b) * rows_total + row];
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) sum += c0 + i < q.chunks ? part[i] : 0.0f;
+    }
+    const int seg = row < p.row_end[0] ? 0 : (row < p.row_end[1] ? 1 : 2);
+    const uint32_t local = row - (seg == 0 ? 0 : p.row_end[seg - 1]);
+    p.y[seg][int64_t(b) * p.y_stride[seg] + local] = sum;
+}
+
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
 }  // namespace
@@ -230,21 +433,60 @@ int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], v
     const uint32_t rows_per_group = kRowsPerWave * kWavesPerGroup;
     const dim3 grid(uint32_t((rows + rows_per_group - 1) / rows_per_group)), block(kWavesPerGroup * kWave);
     hipStream_t st = ctx().stream;
-    // every launch multiplies the weights with up to kMaxBatch input vectors; a larger batch
-    // streams the weights again per group of kMaxBatch (from the last-level cache when the
-    // matrices fit it)
-    for (uint32_t b0 = 0; b0 < batch; b0 += kMaxBatch) {
-        const uint32_t nb = min(batch - b0, uint32_t(kMaxBatch));
+    if (batch > uint32_t(kMaxBatch)) {
+        // a batch of tokens: the matrix cores, kTokTile tokens per launch (the weights come
+        // from the last-level cache after the first launch when the matrices fit it)
+        MatmulTokParams q{};
+        q.chunks = (K + kChunkK - 1) / kChunkK;
+        static bool configured = false;  // the staged inputs exceed the 64 KiB default limit
+        if (!configured) {
+            GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(matmul_q4k_tokens_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(kTokLdsBytes)));
+            configured = true;
+        }
+        // up to kMaxTiles tiles of kTokTile tokens per launch (grid.z), every tile streaming the
+        // weights once (from the last-level cache after the first, when the matrices fit it)
+        constexpr uint32_t kMaxTiles = 8;
+        for (uint32_t b0 = 0; b0 < batch; b0 += kMaxTiles * kTokTile) {
+            const uint32_t nb = min(batch - b0, kMaxTiles * uint32_t(kTokTile));
+            const uint32_t tiles = (nb + kTokTile - 1) / kTokTile;
+            q.tokens = tiles * kTokTile;
+            const size_t need = size_t(q.chunks) * q.tokens * rows * sizeof(float);
+            int rc = ensure_workspace(need);
+            if (rc != GRANITE_HIP_OK) return rc;
+            q.partial = static_cast<float*>(ctx().workspace);
+            q.m = p;
+            q.m.x = static_cast<const float*>(x) + int64_t(b0) * x_stride;
+            q.m.x_stride = x_stride;
+            for (int i = 0; i < 3; i++)
+                if (q.m.y[i]) q.m.y[i] += int64_t(b0) * q.m.y_stride[i];
+            q.m.batch = nb;
+            {
+                KernelTimerScope timer("matmul_q4k_tokens");
+                matmul_q4k_tokens_kernel<<<dim3(uint32_t((rows + kTokRows - 1) / kTokRows), q.chunks, tiles),
+                                           dim3(kTokWaves * kWave), kTokLdsBytes, st>>>(q);
+            }
+            rc = launch_status();
+            if (rc != GRANITE_HIP_OK) return rc;
+            {
+                KernelTimerScope timer("matmul_q4k_merge");
+                matmul_q4k_tokens_merge_kernel<<<dim3(uint32_t((rows + 255) / 256), nb), dim3(256), 0, st>>>(q);
+            }
+            rc = launch_status();
+            if (rc != GRANITE_HIP_OK) return rc;
+        }
+        return GRANITE_HIP_OK;
+    }
+    // up to kMaxBatch input vectors: the vector kernel, one launch
+    {
         MatvecParams q = p;
-        q.x = static_cast<const float*>(x) + int64_t(b0) * x_stride;
-        q.x_stride = nb > 1 ? x_stride : 0;
-        for (int i = 0; i < 3; i++)
-            if (q.y[i]) q.y[i] += int64_t(b0) * q.y_stride[i];
-        q.batch = nb;
+        q.x = static_cast<const float*>(x);
+        q.x_stride = batch > 1 ? x_stride : 0;
+        q.batch = batch;
         KernelTimerScope timer("matvec_q4k");
-        if (nb == 1) matvec_q4k_kernel<1><<<grid, block, 0, st>>>(q);
-        else if (nb == 2) matvec_q4k_kernel<2><<<grid, block, 0, st>>>(q);
-        else matvec_q4k_kernel<4><<<grid, block, 0, st>>>(q);  // 3: the fourth vector repeats the third
+        if (batch == 1) matvec_q4k_kernel<1><<<grid, block, 0, st>>>(q);
+        else matvec_q4k_kernel<2><<<grid, block, 0, st>>>(q);
         int rc = launch_status();
         if (rc != GRANITE_HIP_OK) return rc;
     }

@@ -42,7 +42,10 @@ def _check(oracle, got, x, blocks, what):
 @pytest.mark.parametrize("K,heads,kv_heads,head_dim,batch", [(256, 1, 1, 8, 1), (512, 3, 1, 24, 1),
                                                             (2304, 4, 2, 64, 1), (4096, 32, 8, 128, 1),
                                                             (1024, 5, 1, 64, 2), (2048, 8, 2, 128, 3),
-                                                            (1024, 4, 4, 32, 4), (768, 2, 1, 40, 7)])
+                                                            (1024, 4, 4, 32, 4), (768, 2, 1, 40, 7),
+                                                            # batches of tokens: the matrix-core kernel
+                                                            (256, 1, 1, 8, 5), (4096, 32, 8, 128, 64),
+                                                            (1280, 3, 1, 88, 33), (2048, 8, 2, 128, 32), (512, 2, 2, 16, 300)])
 def test_fused_qkv_matvec_q4k(gpu, oracle, K, heads, kv_heads, head_dim, batch):
     say(f"fused qkv q4k K={K} heads={heads} kv_heads={kv_heads} head_dim={head_dim} batch={batch}")
     case = W.make_qkv_projection(seed=K + heads + batch, K=K, num_heads=heads, num_kv_heads=kv_heads,
