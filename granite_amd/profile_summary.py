@@ -8,8 +8,8 @@ bench.py reads for `roofline.traffic`).
 `collect` runs, per workload, one `rocprofv3 --kernel-trace --stats` pass and one `--pmc`
 pass per counter group (every pass is its own process: rocprofv3 does not split counters
 over passes, and a group holds at most 8 SQ counters), always with `python3 bench.py ...`
-as the profiled program.  Raw output goes to gpurun_out/prof/<workload>/; only the summaries
-are meant to be kept.
+as the profiled program.  Raw output goes to $GRANITE_PROFILE_RAW/<workload>/ (default
+build/prof_raw/, which git ignores); only the summaries are meant to be kept.
 """
 from __future__ import annotations
 
@@ -23,7 +23,7 @@ import sys
 from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent.parent
-RAW = ROOT / "gpurun_out" / "prof"
+RAW = Path(os.environ.get("GRANITE_PROFILE_RAW", ROOT / "build" / "prof_raw")).resolve()
 PROFILES = ROOT / "profiles"
 
 WORKLOADS = ["paged_decode", "prefill", "chunked_prefill", "tree", "decode_contiguous", "rope_append",
