@@ -176,6 +176,7 @@ SIGNATURES = {
     "granite_hip_fused_qkv_matvec_q4k": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32]),
     "granite_hip_fused_qkv_matvec_q4k_batched": (
         _int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _u32, _u32, _u32, _u32]),
+    "granite_hip_q4k_workspace_required": (C.c_size_t, [_u32, C.c_uint64, _u32]),
     "granite_hip_matvec_q4k": (_int, [_vp, _vp, _vp, _u32, _u32]),
     "granite_hip_matvec_q4k_batched": (_int, [_vp, _i64, _vp, _vp, _i64, _u32, _u32, _u32]),
     "granite_hip_workspace_bytes": (C.c_size_t, []),

@@ -592,6 +592,10 @@ int granite_hip_matvec_q4k_batched(const void* x, int64_t x_stride, const void* 
     return ghip::launch_matvec_q4k(x, x_stride, ws, ys, strides, n, K, batch);
 }
 
+size_t granite_hip_q4k_workspace_required(uint32_t K, uint64_t rows, uint32_t batch) {
+    return ghip::matvec_q4k_scratch_bytes(K, rows, batch);
+}
+
 int granite_hip_matvec_q4k(const void* x, const void* w, void* y, uint32_t K, uint32_t N) {
     return granite_hip_matvec_q4k_batched(x, K, w, y, N, K, N, 1);
 }

@@ -107,6 +107,7 @@ int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch
 int launch_attention(const granite_hip_attention_args& a, const ScratchSource& scratch = {});
 int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes);
 int launch_rope_append(const granite_hip_rope_args& a);
+size_t matvec_q4k_scratch_bytes(uint32_t K, uint64_t rows, uint32_t batch);
 int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], void* const y[3],
                       const int64_t y_stride[3], const uint32_t n[3], uint32_t K, uint32_t batch);
 

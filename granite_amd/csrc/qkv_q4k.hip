@@ -406,6 +406,15 @@ inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 
 }  // namespace
 
+// Scratch bytes a projection of `batch` tokens onto `rows` weight rows needs (the chunk sums
+// of the matrix-core path; none for the vector kernel).
+size_t matvec_q4k_scratch_bytes(uint32_t K, uint64_t rows, uint32_t batch) {
+    if (batch <= uint32_t(kMaxBatch) || K == 0) return 0;
+    constexpr uint32_t kMaxTiles = 8;
+    const uint32_t tiles = min((batch + kTokTile - 1) / kTokTile, kMaxTiles);
+    return size_t((K + kChunkK - 1) / kChunkK) * tiles * kTokTile * rows * sizeof(float);
+}
+
 int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], void* const y[3],
                       const int64_t y_stride[3], const uint32_t n[3], uint32_t K, uint32_t batch) {
     if (!x) return GRANITE_HIP_ENULL;
@@ -452,8 +461,7 @@ int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], v
             const uint32_t nb = min(batch - b0, kMaxTiles * uint32_t(kTokTile));
             const uint32_t tiles = (nb + kTokTile - 1) / kTokTile;
             q.tokens = tiles * kTokTile;
-            const size_t need = size_t(q.chunks) * q.tokens * rows * sizeof(float);
-            int rc = ensure_workspace(need);
+            int rc = ensure_workspace(matvec_q4k_scratch_bytes(K, rows, nb));
             if (rc != GRANITE_HIP_OK) return rc;
             q.partial = static_cast<float*>(ctx().workspace);
             q.m = p;

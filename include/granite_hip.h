@@ -432,6 +432,12 @@ int granite_hip_fused_qkv_matvec_q4k_batched(const void *x, int64_t x_stride, co
                                              uint32_t K, uint32_t Nq, uint32_t Nkv,
                                              uint32_t batch);
 
+/* Bytes of library scratch a projection of `batch` tokens onto `rows` weight
+ * rows (Nq + 2 Nkv for the fused form) needs; 0 for up to two tokens.  Reserve
+ * it with granite_hip_reserve_workspace to keep the batched forms from
+ * allocating on their first call. */
+size_t granite_hip_q4k_workspace_required(uint32_t K, uint64_t rows, uint32_t batch);
+
 /* MetalCompute::matvec_q4k (metal_compute.h:73-79; kernel metal_shaders_quant.h:59-163):
  * y[N] = W x, the output projection behind attention (transformer.mm:2650, 2955). */
 int granite_hip_matvec_q4k(const void *x, const void *w, void *y, uint32_t K, uint32_t N);

@@ -107,3 +107,22 @@ def test_rejects_bad_arguments(gpu):
     assert lib.granite_hip_matvec_q4k(buf.ptr + 4, buf.ptr, buf.ptr, 256, 4) == _capi.EINVAL  # alignment
     assert lib.granite_hip_matvec_q4k(buf.ptr, buf.ptr, buf.ptr, 256, 0) == _capi.OK
     gpu.sync()
+
+
+def test_batched_projection_scratch_can_be_reserved(gpu, oracle):
+    """The matrix-core path keeps its chunk sums in library scratch: the stated requirement,
+    reserved once, is enough (no growth during the call)."""
+    lib = _capi.load()
+    case = W.make_qkv_projection(seed=77, K=1024, num_heads=4, num_kv_heads=2, head_dim=64, batch=40)
+    rows = case.Nq + 2 * case.Nkv
+    assert lib.granite_hip_q4k_workspace_required(case.K, rows, 2) == 0
+    need = lib.granite_hip_q4k_workspace_required(case.K, rows, 40)
+    assert need == 2 * 64 * rows * 4        # two chunks of K, two tiles of 32 tokens
+    gpu.reserve_workspace(need)
+    held = gpu.workspace_bytes()
+    yq, yk, yv = (dev(np.zeros((40, n), np.float32)) for n in (case.Nq, case.Nkv, case.Nkv))
+    gpu.fused_qkv_matvec_q4k(dev(case.x), dev(case.wq), dev(case.wk), dev(case.wv), yq, yk, yv, case.K, case.Nq,
+                             case.Nkv, batch=40)
+    gpu.sync()
+    assert gpu.workspace_bytes() == held
+    _check(oracle, yq.read(np.float32, (40, case.Nq)), case.x, case.wq, "yq")
