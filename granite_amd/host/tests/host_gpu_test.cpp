@@ -31,6 +31,7 @@ void go_attention_paged(const float* q, const uint16_t* pool_k, const uint16_t* 
                         const int32_t* table, int block_size, float* context, float* lse, int batch,
                         int seq_len, int num_heads, int num_kv_heads, int head_dim, int total_seq,
                         int start_pos, float scale);
+void go_matvec_q4k(const float* x, const uint8_t* W, float* y, int K, int N, int batch);
 void go_attention_cached(const float* q, const uint16_t* cache_k, const uint16_t* cache_v,
                          float* context, float* lse, int batch, int seq_len, int num_heads,
                          int num_kv_heads, int head_dim, int total_seq, int max_seq,
@@ -918,6 +919,76 @@ TEST_CASE(chunked_prefill_driver) {
         d3.finish();
         CHECK(cache.seq_len() == n);
     }
+}
+
+
+// The projections either side of attention through HipCompute (MetalCompute::
+// fused_qkv_matvec_q4k and matvec_q4k, include/granite/metal_compute.h:683-694, 73-79), one
+// token and a batch of tokens, against the oracle's dequantise-and-multiply; and the scratch
+// the batched form needs, reserved up front.
+TEST_CASE(hip_compute_q4k_projections) {
+    REQUIRE(backend() != nullptr);
+    HipCompute* hc = get_hip_compute();
+    REQUIRE(hc != nullptr);
+    const int K = 1024, Nq = 256, Nkv = 64, batch = 40, blocks = K / 256;
+    // random Q4_K super-blocks: any 144 bytes are a valid block once d and dmin are small halves
+    std::mt19937 gen(4242);
+    auto make_weights = [&](int rows) {
+        std::vector<uint8_t> w(size_t(rows) * blocks * 144);
+        for (auto& b : w) b = uint8_t(gen());
+        for (size_t blk = 0; blk < w.size() / 144; ++blk) {
+            const uint16_t d = go_fp32_to_fp16(3e-4f + 1e-6f * float(gen() % 400));
+            const uint16_t dmin = go_fp32_to_fp16(2e-4f + 1e-6f * float(gen() % 400));
+            std::memcpy(&w[blk * 144], &d, 2);
+            std::memcpy(&w[blk * 144 + 2], &dmin, 2);
+        }
+        return w;
+    };
+    auto wq = make_weights(Nq), wk = make_weights(Nkv), wv = make_weights(Nkv);
+    auto x = randn(size_t(batch) * K, 99);
+    Tensor X = upload({batch, K}, DataType::FP32, x);
+    Tensor WQ = upload({int64_t(wq.size())}, DataType::UINT8, wq);
+    Tensor WK = upload({int64_t(wk.size())}, DataType::UINT8, wk);
+    Tensor WV = upload({int64_t(wv.size())}, DataType::UINT8, wv);
+    Tensor YQ = Tensor::allocate({batch, Nq}, DataType::FP32, backend()).take();
+    Tensor YK = Tensor::allocate({batch, Nkv}, DataType::FP32, backend()).take();
+    Tensor YV = Tensor::allocate({batch, Nkv}, DataType::FP32, backend()).take();
+    auto ptr = [&](const Tensor& t) { return hip_device_pointer(backend(), t.buffer()); };
+
+    auto check = [&](const Tensor& Y, const std::vector<uint8_t>& w, int N, int rows, const char* what) {
+        std::vector<float> want(size_t(rows) * N);
+        go_matvec_q4k(x.data(), w.data(), want.data(), K, N, rows);
+        auto got = download<float>(Y);
+        double worst = 0, scale = 0;
+        for (size_t i = 0; i < want.size(); ++i) {
+            worst = std::max(worst, std::fabs(double(got[i]) - double(want[i])));
+            scale = std::max(scale, std::fabs(double(want[i])));
+        }
+        std::printf("  %s: max abs err %.3g (values up to %.3g)\n", what, worst, scale);
+        CHECK(worst <= 1e-4 * std::max(scale, 1.0));  // float sums of K = 1024 products, two orders
+    };
+    // one token: the reference's signature
+    CHECK_OK(hc->fused_qkv_matvec_q4k(ptr(X), ptr(WQ), ptr(WK), ptr(WV), ptr(YQ), ptr(YK), ptr(YV), K, Nq, Nkv));
+    hc->sync();
+    check(YQ, wq, Nq, 1, "fused qkv, one token (q)");
+    check(YV, wv, Nkv, 1, "fused qkv, one token (v)");
+    CHECK_OK(hc->matvec_q4k(ptr(X), ptr(WK), ptr(YK), K, Nkv));
+    hc->sync();
+    check(YK, wk, Nkv, 1, "matvec");
+    // a batch of tokens, its scratch reserved first
+    const size_t need = granite_hip_q4k_workspace_required(K, Nq + 2 * Nkv, batch);
+    CHECK(need > 0);
+    CHECK_OK(hc->reserve_workspace(need));
+    const size_t held = hc->workspace_bytes();
+    CHECK_OK(hc->fused_qkv_matvec_q4k_batched(ptr(X), ptr(WQ), ptr(WK), ptr(WV), ptr(YQ), ptr(YK), ptr(YV), K, Nq,
+                                              Nkv, batch));
+    hc->sync();
+    CHECK(hc->workspace_bytes() == held);
+    check(YQ, wq, Nq, batch, "fused qkv, 40 tokens (q)");
+    check(YK, wk, Nkv, batch, "fused qkv, 40 tokens (k)");
+    check(YV, wv, Nkv, batch, "fused qkv, 40 tokens (v)");
+    CHECK_CODE(hc->matvec_q4k(ptr(X), ptr(WK), ptr(YK), 300, Nkv), ErrorCode::InvalidArgument);  // K % 256
+    for (Tensor* t : {&X, &WQ, &WK, &WV, &YQ, &YK, &YV}) backend()->destroy_buffer(t->buffer());
 }
 
 
