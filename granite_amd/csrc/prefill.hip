@@ -73,7 +73,7 @@
 // Algorithmic work: 4 * D flops per visible (query, key) pair.
 #include <cstdlib>
 
-#include "common.h"
+#include "prefill_shared.h"
 
 namespace ghip {
 namespace {
@@ -99,43 +99,6 @@ struct Geometry {
     static constexpr int kBlocks = kD / 32;  // 32-row head-dim blocks of O^T; also 64-byte chunks of a V row
     static constexpr int kPhase = kSteps + 2 * kBlocks;  // MFMAs of a pipeline phase
 };
-constexpr float kNegBig = -1.0e30f;
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
-constexpr uint32_t kMaxFusedNodes = 256;  // largest tree whose ancestor mask a workgroup builds itself
-constexpr float kProbLimit = 16384.0f;  // a row's probabilities of a sub-tile may sum to this much
-
-enum : int { kRowsContiguous = 0, kRowsPagedPow2 = 1, kRowsPagedAny = 2 };
-
-struct AttnParams {
-    const void* q;
-    void* out;
-    float* lse;
-    int64_t q_tok_stride, q_head_stride, out_tok_stride, out_head_stride;
-    const uint16_t* k;
-    const uint16_t* v;
-    const int32_t* table;
-    uint32_t block_size;
-    int bs_shift;
-    int64_t a_tok_stride, a_head_stride;
-    uint32_t cache_len;
-    const uint16_t* k_extra;
-    const uint16_t* v_extra;
-    uint32_t extra_len;
-    const uint32_t* tree_mask;      // ancestor bit matrix in memory (trees beyond kMaxFusedNodes)
-    const int32_t* tree_parents;    // or: parent pointers, the workgroup builds its own matrix in LDS
-    uint32_t mask_words;
-    int mask_mode;
-    uint32_t start_pos, seq_q, num_heads, group;
-    float scale_log2;
-    uint32_t q_tiles, n_splits;  // the grid: q_tiles * num_heads * n_splits workgroups
-    // split-K over the key tiles (n_splits > 1): unnormalised partial results
-    float* part_o;   // [split, head, q, D]
-    float* part_ml;  // [split, head, q, 2] = (reference max, sum)
-    void* final_out;
-    int64_t final_tok_stride, final_head_stride;
-};
-
 __device__ __forceinline__ half8 as_half8(uint4v x) { return __builtin_bit_cast(half8, x); }
 
 // Row of the K/V array that holds key `idx`: of the cache segment (through the
@@ -1039,11 +1002,17 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     const int rows = !a.block_table ? kRowsContiguous
                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
+    // The wide-row kernel (prefill_wide.hip) where it applies: head size 128, half queries,
+    // no extra key segment, contiguous rows or blocks of a power of two >= 8 tokens.
+    bool wide = D == 128 && !qf32 && a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE &&
+                rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3);
+    if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) wide = wide && e[0] != 't';  // "tiles"
     int rc;
     {
         KernelTimerScope timer("attention_tiles");
-        rc = D == 128 ? launch_tiles_types<128>(p, grid, rows, qf32, of32)
-                      : launch_tiles_types<64>(p, grid, rows, qf32, of32);
+        if (wide) rc = launch_tiles_wide(p, grid, of32);
+        else rc = D == 128 ? launch_tiles_types<128>(p, grid, rows, qf32, of32)
+                           : launch_tiles_types<64>(p, grid, rows, qf32, of32);
     }
     if (rc != GRANITE_HIP_OK || n_splits == 1) return rc;
     {
