@@ -211,7 +211,7 @@ def bench_prefill(gpu, steps, warmup, cpu):
         "dtype": "f16 MFMA, f32 accumulate", "kernels_ms": {k: round(v[0], 4) for k, v in kern.items()},
     }
     res["roofline"] = roofline("mfma", flops, kern["attention_tiles"][0], profiled_traffic("prefill", res["workload"]))
-    res["roofline"]["kernel"] = "attention_tiles_kernel"
+    res["roofline"]["kernel"] = "attention_tiles_dma_kernel"
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()
@@ -262,7 +262,7 @@ def bench_chunked_prefill(gpu, steps, warmup, cpu):
     }
     res["roofline"] = roofline("mfma", flops, kern["attention_tiles"][0],
                                profiled_traffic("chunked_prefill", res["workload"]))
-    res["roofline"]["kernel"] = "attention_tiles_kernel"
+    res["roofline"]["kernel"] = "attention_tiles_dma_kernel"
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()

@@ -18,7 +18,7 @@ HOST = PKG / "host"
 LIBDIR = PKG / "lib"
 BINDIR = PKG / "bin"
 
-HIP_SOURCES = ["capi.hip", "kv_ops.hip", "rope.hip", "qkv_q4k.hip", "decode.hip", "decode_stream.hip", "prefill.hip", "prefill_wide.hip"]
+HIP_SOURCES = ["capi.hip", "kv_ops.hip", "rope.hip", "qkv_q4k.hip", "decode.hip", "decode_stream.hip", "prefill.hip", "prefill_dma.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -1002,15 +1002,15 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     const int rows = !a.block_table ? kRowsContiguous
                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
-    // The wide-row kernel (prefill_wide.hip) where it applies: head size 128, half queries,
+    // The direct-to-LDS kernel (prefill_dma.hip) where it applies: head size 128, half queries,
     // no extra key segment, contiguous rows or blocks of a power of two >= 8 tokens.
-    bool wide = D == 128 && !qf32 && a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE &&
+    bool dma = D == 128 && !qf32 && a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE &&
                 rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3);
-    if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) wide = wide && e[0] != 't';  // "tiles"
+    if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) dma = dma && e[0] != 't';  // "tiles": the register-staged kernel
     int rc;
     {
         KernelTimerScope timer("attention_tiles");
-        if (wide) rc = launch_tiles_wide(p, grid, of32);
+        if (dma) rc = launch_tiles_dma(p, grid, of32);
         else rc = D == 128 ? launch_tiles_types<128>(p, grid, rows, qf32, of32)
                            : launch_tiles_types<64>(p, grid, rows, qf32, of32);
     }

@@ -39,9 +39,13 @@
 // half queries, no extra key segment (no tree mask), contiguous cache or paged cache with a
 // power-of-two block size >= 8.
 //
-// kRB, the number of 32-row blocks a wave owns, is 1.  With 2 (four waves of 64 rows, one per
-// SIMD) an LDS operand read would feed two MFMAs; that form needs about 330 registers per
-// lane and the compiler does not produce it without spilling.
+// kRB, the number of 32-row blocks a wave owns, is 1.  With 2 (-DGHIP_DMA_RB=2: four waves of
+// 64 rows, one per SIMD) an LDS operand read feeds two MFMAs; that form needs 434 registers per
+// lane, the compiler keeps every MFMA result in accumulation registers and moves scores and
+// probabilities between the two register files with about two extra vector instructions per
+// MFMA, and it measured slower (chunked prefill 525 against 506 us on the same box, the causal
+// prefill 68 against 52 us: there a wave then owns a SIMD and the longest row block's walk is
+// not shared).
 //
 // Algorithmic work: 4 * D flops per visible (query, key) pair.
 #include <type_traits>
@@ -52,7 +56,10 @@ namespace ghip {
 namespace {
 
 constexpr int kD = 128;
-constexpr int kRB = 1;          // 32-row blocks per wave
+#ifndef GHIP_DMA_RB
+#define GHIP_DMA_RB 1
+#endif
+constexpr int kRB = GHIP_DMA_RB;  // 32-row blocks per wave
 constexpr int kWaves = 8 / kRB;
 constexpr int kWBM = 256;       // query rows per workgroup
 constexpr int kWBN = 64;        // keys per tile
@@ -65,7 +72,7 @@ constexpr uint32_t kVTile = kWBN * kD * 2;    // 16384
 constexpr uint32_t kVRegion = kStages * kKTile;
 constexpr uint32_t kEntryRegion = kStages * (kKTile + kVTile);  // 139264
 constexpr uint32_t kEntries = 64;  // block-table entries a wave keeps in LDS: those of its next 64 tiles
-constexpr size_t kWideLds = kEntryRegion + size_t(kWaves) * kEntries * sizeof(uint32_t);
+constexpr size_t kDmaLds = kEntryRegion + size_t(kWaves) * kEntries * sizeof(uint32_t);
 constexpr int kSteps = kD / 16;   // MFMAs of the scores of a sub-tile and row block
 constexpr int kBlocks = kD / 32;  // 32-row head-dim blocks of O^T
 constexpr int kSlots = 2 * kRB * kSteps;  // MFMAs of a phase; side work is issued after each
@@ -99,14 +106,14 @@ __device__ __forceinline__ void dma_lanes(uint32_t lds_addr, const void* addr) {
 // are scarcest.  Nothing reads an output block with a vector instruction inside the loop
 // except the rare rescale, which waits first (mfma_drain).
 __device__ __forceinline__ void mfma_output(float16v& o, const uint4v& a, const half8& b) {
-#ifdef GHIP_WIDE_TIED_OUTPUT
+#ifdef GHIP_DMA_TIED_OUTPUT
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(o) : "v"(a), "v"(b));
 #else
     o = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(a), b, o, 0, 0, 0);
 #endif
 }
 __device__ __forceinline__ void mfma_drain() {
-#ifdef GHIP_WIDE_TIED_OUTPUT
+#ifdef GHIP_DMA_TIED_OUTPUT
     asm volatile("s_nop 15\n\ts_nop 15");
 #endif
 }
@@ -116,7 +123,7 @@ __device__ __forceinline__ void wait_transfers() {
 }
 
 template <bool kOutF32, bool kPaged>
-__global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_wide_kernel(AttnParams p) {
+__global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
     const uint32_t lds0 = uint32_t(uintptr_t((lds_byte*)s_raw));  // LDS address of the tile buffers
 
@@ -390,7 +397,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_wide_kernel(Attn
     auto fused_phase = [&](auto kb, auto sub_q, auto vb, auto sub_v, bool masked, bool softmax_live, uint32_t j_q,
                            float16v (&s_out)[kRB], const float16v (&s_in)[kRB], half8 (&p_out)[kRB][2],
                            const half8 (&p_prev)[kRB][2], auto&& side) __attribute__((always_inline)) {
-        constexpr int kRing = 3;
+#ifndef GHIP_DMA_RING
+#define GHIP_DMA_RING 3
+#endif
+        constexpr int kRing = GHIP_DMA_RING;
         uint4v ring[kRing];
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(kb, sub_q, i);
@@ -449,11 +459,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_wide_kernel(Attn
             p_out[rb][0] = as_half8(uint4v{pw[rb][0], pw[rb][1], pw[rb][2], pw[rb][3]});
             p_out[rb][1] = as_half8(uint4v{pw[rb][4], pw[rb][5], pw[rb][6], pw[rb][7]});
             if (softmax_live) {
-#ifdef EXP_NOREBASE
-                if (false) {
-#else
                 if (__any(!(psum[rb] < kProbLimit))) {  // rare: the reference has to move, redo the sub-tile
-#endif
                     rebase(rb, s_in[rb]);
                     psum[rb] = probabilities_once(rb, s_in[rb], p_out[rb]);
                 }
@@ -548,8 +554,12 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_wide_kernel(Attn
             const uint32_t j = 2 * it;
             fused_phase(IC<B>{}, IC<1>{}, IC<(B + 3) & 3>{}, IC<1>{}, j + 1 >= j_mask, j < j_end, j + 1, s1, s0,
                         p_new, p_old, [&](int slot) __attribute__((always_inline)) {
-                            if (slot == 1) stage_next(it, (B + 3) & 3, (B + 2) & 3, 0);
-                            if (slot == 3) stage_next(it, (B + 3) & 3, (B + 2) & 3, 1);
+#ifndef GHIP_DMA_SLOT_V
+#define GHIP_DMA_SLOT_V 9
+#define GHIP_DMA_SLOT_K 11
+#endif
+                            if (slot == GHIP_DMA_SLOT_V) stage_next(it, (B + 3) & 3, (B + 2) & 3, 0);
+                            if (slot == GHIP_DMA_SLOT_K) stage_next(it, (B + 3) & 3, (B + 2) & 3, 1);
                         });
             fused_phase(IC<(B + 1) & 3>{}, IC<0>{}, IC<B>{}, IC<0>{}, j + 2 >= j_mask, j + 1 < j_end, j + 2, s0, s1,
                         p_old, p_new, [](int) {});
@@ -643,27 +653,27 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_wide_kernel(Attn
 }
 
 template <bool kOutF32, bool kPaged>
-int launch_wide(const AttnParams& p, dim3 grid) {
-    auto kernel = attention_wide_kernel<kOutF32, kPaged>;
+int launch_dma(const AttnParams& p, dim3 grid) {
+    auto kernel = attention_tiles_dma_kernel<kOutF32, kPaged>;
     static bool configured = false;  // the tile buffers exceed the 64 KiB default limit
     if (!configured) {
         GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kWideLds)));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDmaLds)));
         configured = true;
     }
-    kernel<<<grid, dim3(kWThreads), kWideLds, ctx().stream>>>(p);
+    kernel<<<grid, dim3(kWThreads), kDmaLds, ctx().stream>>>(p);
     return launch_status();
 }
 
 }  // namespace
 
-size_t tiles_wide_lds_bytes() { return kWideLds; }
+size_t tiles_dma_lds_bytes() { return kDmaLds; }
 
-int launch_tiles_wide(const AttnParams& p, dim3 grid, bool out_f32) {
+int launch_tiles_dma(const AttnParams& p, dim3 grid, bool out_f32) {
     const bool paged = p.table != nullptr;
     if (paged && (p.bs_shift < 3)) return GRANITE_HIP_EUNSUPPORTED;
-    if (out_f32) return paged ? launch_wide<true, true>(p, grid) : launch_wide<true, false>(p, grid);
-    return paged ? launch_wide<false, true>(p, grid) : launch_wide<false, false>(p, grid);
+    if (out_f32) return paged ? launch_dma<true, true>(p, grid) : launch_dma<true, false>(p, grid);
+    return paged ? launch_dma<false, true>(p, grid) : launch_dma<false, false>(p, grid);
 }
 
 }  // namespace ghip

@@ -1,5 +1,5 @@
 // Declarations shared by the two prefill kernel files: the launch parameters that
-// launch_attention() fills in, the softmax constants, and the launcher of the wide-row kernel.
+// launch_attention() fills in, the softmax constants, and the launcher of the direct-to-LDS kernel.
 #pragma once
 
 #include "common.h"
@@ -43,11 +43,11 @@ struct AttnParams {
     int64_t final_tok_stride, final_head_stride;
 };
 
-// The wide-row form of the tiles kernel (prefill_wide.hip): same grid, same partial-result
+// The direct-to-LDS form of the tiles kernel (prefill_dma.hip): same grid, same partial-result
 // layout and same merge launch as attention_tiles_kernel.  Only for head size 128, half
 // queries, no extra key segment, and a contiguous cache or a paged one whose block size is a
 // power of two of at least 8 tokens; the caller checks that.
-int launch_tiles_wide(const AttnParams& p, dim3 grid, bool out_f32);
-size_t tiles_wide_lds_bytes();
+int launch_tiles_dma(const AttnParams& p, dim3 grid, bool out_f32);
+size_t tiles_dma_lds_bytes();
 
 }  // namespace ghip

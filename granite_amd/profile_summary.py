@@ -29,8 +29,8 @@ PROFILES = ROOT / "profiles"
 WORKLOADS = ["paged_decode", "prefill", "chunked_prefill", "tree", "decode_contiguous", "rope_append",
              "qkv_q4k", "copy_calibration"]
 MFMA_BOUND = {"prefill", "chunked_prefill"}
-DOMINANT = {"paged_decode": "decode_stream_kernel", "prefill": "attention_tiles_kernel",
-            "chunked_prefill": "attention_tiles_kernel", "tree": "attention_tiles_kernel",
+DOMINANT = {"paged_decode": "decode_stream_kernel", "prefill": "attention_tiles_dma_kernel",
+            "chunked_prefill": "attention_tiles_dma_kernel", "tree": "attention_tiles_kernel",
             "decode_contiguous": "decode_splitk_kernel", "rope_append": "rope_append_kernel",
             "qkv_q4k": "matvec_q4k_kernel", "copy_calibration": "kv_gather_kernel"}
 
@@ -190,7 +190,8 @@ def summarise(workloads: list[str]) -> int:
         if "roofline" in res:
             L += ["", f"Roofline from the event timing: `{json.dumps(res['roofline'])}`"]
         L += ["", "## Registers, LDS, scratch (kernel trace; LDS is the static part, the K/V tile buffers of "
-              "`attention_tiles_kernel` are 101376 B of dynamic LDS on top)", "",
+              "`attention_tiles_dma_kernel` are 141312 B and those of `attention_tiles_kernel` 101376 B of "
+              "dynamic LDS on top)", "",
               "| kernel | VGPRs | AGPRs | SGPRs | LDS bytes | scratch bytes | workgroup |", "|---|---|---|---|---|---|---|"]
         for k, v in sorted(resources(w).items()):
             L.append(f"| `{k[:70]}` | " + " | ".join(v) + " |")
