@@ -412,10 +412,12 @@ def bench_mfma_calibration(gpu, steps, warmup, cpu):
     measurement aid beside the attention library): zeros (the part keeps its peak clock)
     against normally distributed fp16 values (the power limit holds the clock down), both MFMA
     shapes, and then with the other instructions an attention inner loop issues per MFMA
-    beside them -- float FMAs, an exponential, a 16-byte LDS operand read -- with one and with
-    two waves per SIMD.  The last line of the mix table (3 FMAs, 1 exponential, 1 LDS read) is
-    the prefill kernel's mix: the rate an MFMA-bound attention kernel can be compared with
-    beside the published peak.  Not part of `--workload all`."""
+    beside them -- float FMAs, exponentials, 16-byte LDS operand reads, scalar instructions --
+    with one and with two waves per SIMD.  The mixes are given per pair of MFMAs; two of them
+    are what the hardware counters report for the two prefill kernels (profiles/
+    chunked_prefill.md: vector, LDS and scalar instructions per MFMA), so the rate of such a
+    row is what that kernel's instruction mix leaves of the matrix cores with no tile staging,
+    no barrier and no masks.  Not part of `--workload all`."""
     from granite_amd import DeviceBuffer, calibration
     rng = np.random.default_rng(11)
     n = 1 << 20
@@ -424,22 +426,28 @@ def bench_mfma_calibration(gpu, steps, warmup, cpu):
     bufs = {k: DeviceBuffer.from_numpy(v) for k, v in data.items()}
     iterations = 20000
 
-    def rate(kind, shape, waves, mix):
+    def rate(kind, shape, waves, per_pair):
         best = 0.0
         for _ in range(max(1, min(steps, 3))):
-            flops, ms = calibration.mfma_rate(bufs[kind], n, iterations, shape=shape, waves_per_simd=waves, mix=mix)
+            flops, ms = calibration.mfma_mix(bufs[kind], n, iterations, shape=shape, waves_per_simd=waves,
+                                             per_pair=per_pair)
             best = max(best, flops / (ms * 1e-3) / 1e12)
         return round(best, 1)
 
-    rates = {f"{kind}_{shape}": rate(kind, shape, 2, (0, 0, 0)) for kind in data for shape in (32, 16)}
-    mixes = {"mfma_only": (0, 0, 0), "4_fma": (4, 0, 0), "8_fma": (8, 0, 0), "1_exp": (0, 1, 0),
-             "3_fma_1_exp": (3, 1, 0), "1_lds_read": (0, 0, 1), "3_fma_1_exp_1_lds_read": (3, 1, 1)}
+    rates = {f"{kind}_{shape}": rate(kind, shape, 2, (0, 0, 0, 0)) for kind in data for shape in (32, 16)}
+    mixes = {"mfma_only": (0, 0, 0, 0), "4_fma": (8, 0, 0, 0), "8_fma": (16, 0, 0, 0), "1_exp": (0, 2, 0, 0),
+             "3_fma_1_exp": (6, 2, 0, 0), "1_lds_read": (0, 0, 2, 0), "3_fma_1_exp_1_lds_read": (6, 2, 2, 0),
+             "3_fma_1_exp_half_lds_read": (6, 2, 1, 0),
+             "tiles_dma_kernel_mix_3_fma_1_exp_1.5_lds_2_salu": (6, 2, 3, 4),
+             "tiles_kernel_mix_4_fma_1_exp_1.5_lds_3_salu": (8, 2, 3, 6),
+             "rows64_mix_3.5_fma_1_exp_0.5_lds_1.5_salu": (7, 2, 1, 3)}
     mix_rates = {name: {f"{w}_wave_per_simd": rate("normal", 32, w, mix) for w in (1, 2)}
                  for name, mix in mixes.items()}
     return {"workload": "mfma_calibration_register_operands_one_workgroup_per_cu", "metric": "mfma_TFLOPs",
             "unit": "TFLOP/s", "value": rates["normal_32"], "ms_per_step": 0.0,
             "rates_TFLOPs": {"zeros_32x32x16": rates["zeros_32"], "zeros_16x16x32": rates["zeros_16"],
                              "normal_32x32x16": rates["normal_32"], "normal_16x16x32": rates["normal_16"]},
+            "instruction_mix_per_pair_of_mfma": {k: list(v) for k, v in mixes.items()},
             "instruction_mix_TFLOPs_32x32x16_normal": mix_rates,
             "peak_TFLOPs": 2500.0}
 

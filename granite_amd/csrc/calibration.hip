@@ -7,7 +7,9 @@
 // held back by its power limit.  The mix form adds, after every MFMA, what an attention
 // inner loop issues beside it -- a few float FMAs, an exponential, a 16-byte LDS read per
 // lane whose data feeds a later MFMA -- and so measures what the instruction mix itself
-// leaves of the matrix cores, with no staging, no barriers and no loop bookkeeping.
+// leaves of the matrix cores, with no staging, no barriers and no loop bookkeeping.  The mix
+// is given per pair of MFMAs, so that half an instruction per MFMA (an LDS operand that feeds
+// two MFMAs) can be expressed, and may include scalar instructions.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -31,7 +33,9 @@ constexpr size_t kLdsBytes = 100 * 1024;        // and enough LDS to keep one wo
     } while (0)
 
 // kWide: 32x32x16 (16 MFMAs a pass) or 16x16x32 (32 MFMAs a pass, the same flops).
-template <bool kWide, int kFma, int kExp, int kLds>
+// kFma, kExp, kLds, kSalu: instructions per PAIR of MFMAs; the first MFMA of a pair is followed
+// by the larger half of each.
+template <bool kWide, int kFma, int kExp, int kLds, int kSalu>
 __global__ void __launch_bounds__(512, 1)
     mfma_rate_kernel(const uint4v* __restrict__ operands, uint32_t n_vec, uint32_t iterations,
                      float* sink) {
@@ -69,20 +73,29 @@ __global__ void __launch_bounds__(512, 1)
 #pragma unroll
         for (int i = 0; i < 4; i++) ld[i] = __builtin_bit_cast(uint4v, a[i]);
         const uint4v* lp = s_operands + lane;  // 64 lanes x 16 bytes: every bank once
+        uint32_t scalar = iterations;
         for (uint32_t it = 0; it < iterations; it++) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
+                const bool second = r & 1;  // of the pair
                 const half8 aa = kLds > 0 ? __builtin_bit_cast(half8, ld[r & 3]) : a[r & 3];
                 c[r & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aa, b[(r + (r >> 2)) & 3], c[r & 3], 0, 0, 0);
 #pragma unroll
-                for (int j = 0; j < kLds; j++) ld[(r + 2) & 3] = lp[64 * ((r + j + it) & 15)];  // used two MFMAs on
+                for (int j = 0; j < (second ? kLds / 2 : (kLds + 1) / 2); j++)
+                    ld[(r + 2 + j) & 3] = lp[64 * ((r + j + it) & 15)];  // used two MFMAs on
 #pragma unroll
-                for (int j = 0; j < kFma; j++) x[(r + j) & 7] = __builtin_fmaf(x[(r + j) & 7], 0.999f, 0.001f);
+                for (int j = 0; j < (second ? kFma / 2 : (kFma + 1) / 2); j++)
+                    x[(r + j) & 7] = __builtin_fmaf(x[(r + j) & 7], 0.999f, 0.001f);
 #pragma unroll
-                for (int j = 0; j < kExp; j++) e[(r + j) & 3] = __builtin_amdgcn_exp2f(e[(r + j) & 3] * 0.5f);
+                for (int j = 0; j < (second ? kExp / 2 : (kExp + 1) / 2); j++)
+                    e[(r + j) & 3] = __builtin_amdgcn_exp2f(e[(r + j) & 3] * 0.5f);
+#pragma unroll
+                for (int j = 0; j < (second ? kSalu / 2 : (kSalu + 1) / 2); j++)
+                    asm volatile("s_add_u32 %0, %0, 3" : "+s"(scalar));
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        total += float(scalar & 1);
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -108,10 +121,10 @@ __global__ void __launch_bounds__(512, 1)
     if (total == 1.2345e-30f) sink[0] = total;  // keeps the loop alive; practically never taken
 }
 
-template <bool kWide, int kFma, int kExp, int kLds>
+template <bool kWide, int kFma, int kExp, int kLds, int kSalu>
 int run(const uint4v* operands, uint32_t n_vec, uint32_t iterations, uint32_t workgroups, uint32_t threads,
         float* sink, float* milliseconds) {
-    auto kernel = mfma_rate_kernel<kWide, kFma, kExp, kLds>;
+    auto kernel = mfma_rate_kernel<kWide, kFma, kExp, kLds, kSalu>;
     CAL_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
     hipEvent_t start, stop;
@@ -131,10 +144,10 @@ int run(const uint4v* operands, uint32_t n_vec, uint32_t iterations, uint32_t wo
 
 }  // namespace
 
-extern "C" int granite_hip_cal_mfma_rate(int device, const void* operands_f16, uint64_t n_halves,
-                                         uint32_t iterations, int shape, int waves_per_simd,
-                                         int fma_per_mfma, int exp_per_mfma, int lds_reads_per_mfma,
-                                         double* flops, float* milliseconds) {
+extern "C" int granite_hip_cal_mfma_mix(int device, const void* operands_f16, uint64_t n_halves,
+                                        uint32_t iterations, int shape, int waves_per_simd,
+                                        int fma_per_pair, int exp_per_pair, int lds_reads_per_pair,
+                                        int salu_per_pair, double* flops, float* milliseconds) {
     if (!operands_f16 || !flops || !milliseconds) return -1;
     if (n_halves < kLdsHalves || n_halves % 8 != 0 || n_halves / 8 > 0xFFFFFFFFull) return -1;
     if (iterations == 0 || iterations > (1u << 20)) return -1;
@@ -148,18 +161,35 @@ extern "C" int granite_hip_cal_mfma_rate(int device, const void* operands_f16, u
     CAL_CHECK(hipMalloc(&sink, 256));
     const auto* ops = static_cast<const uint4v*>(operands_f16);
     const uint32_t n_vec = uint32_t(n_halves / 8);
-    const int mix = fma_per_mfma * 100 + exp_per_mfma * 10 + lds_reads_per_mfma;
+    const int mix = fma_per_pair * 1000 + exp_per_pair * 100 + lds_reads_per_pair * 10 + salu_per_pair;
     int rc = -1;
-    if (shape == 16 && mix == 0) rc = run<false, 0, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 0) rc = run<true, 0, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 400) rc = run<true, 4, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 800) rc = run<true, 8, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 10) rc = run<true, 0, 1, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 310) rc = run<true, 3, 1, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 1) rc = run<true, 0, 0, 1>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 32 && mix == 311) rc = run<true, 3, 1, 1>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
+#define GHIP_CAL_MIX(f, e, l, sa)                                                                          \
+    if (shape == 32 && mix == (f) * 1000 + (e) * 100 + (l) * 10 + (sa))                                    \
+        rc = run<true, f, e, l, sa>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
+    if (shape == 16 && mix == 0) rc = run<false, 0, 0, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
+    GHIP_CAL_MIX(0, 0, 0, 0)
+    GHIP_CAL_MIX(8, 0, 0, 0)   // 4 float FMAs per MFMA
+    GHIP_CAL_MIX(16, 0, 0, 0)  // 8
+    GHIP_CAL_MIX(0, 2, 0, 0)   // 1 exponential
+    GHIP_CAL_MIX(6, 2, 0, 0)   // 3 FMAs + 1 exponential
+    GHIP_CAL_MIX(0, 0, 2, 0)   // 1 LDS read
+    GHIP_CAL_MIX(6, 2, 2, 0)   // 3 FMAs + 1 exponential + 1 LDS read
+    GHIP_CAL_MIX(6, 2, 1, 0)   // ... + half an LDS read (an operand feeding two MFMAs)
+    GHIP_CAL_MIX(6, 2, 3, 4)   // what attention_tiles_dma_kernel issues: 3 + 1 vector, 1.5 LDS, 2 scalar
+    GHIP_CAL_MIX(8, 2, 3, 6)   // what attention_tiles_kernel issues: 4 + 1 vector, 1.5 LDS, 3 scalar
+    GHIP_CAL_MIX(7, 2, 1, 3)   // a 64-rows-per-wave form of the former: 3.5 + 1 vector, 0.5 LDS, 1.5 scalar
+#undef GHIP_CAL_MIX
     (void)hipFree(sink);
     // 16 MFMAs of 2 * 32 * 32 * 16 flops (or 32 of half that) per pass and wave
     *flops = double(workgroups) * (threads / kWave) * double(iterations) * 16.0 * 2.0 * 32 * 32 * 16;
     return rc;
+}
+
+extern "C" int granite_hip_cal_mfma_rate(int device, const void* operands_f16, uint64_t n_halves,
+                                         uint32_t iterations, int shape, int waves_per_simd,
+                                         int fma_per_mfma, int exp_per_mfma, int lds_reads_per_mfma,
+                                         double* flops, float* milliseconds) {
+    return granite_hip_cal_mfma_mix(device, operands_f16, n_halves, iterations, shape, waves_per_simd,
+                                    2 * fma_per_mfma, 2 * exp_per_mfma, 2 * lds_reads_per_mfma, 0, flops,
+                                    milliseconds);
 }

@@ -5,6 +5,10 @@ bench.py reads for `roofline.traffic`).
     python -m granite_amd.profile_summary collect [workload ...]    # on the GPU box
     python -m granite_amd.profile_summary summarise [workload ...]  # anywhere, from the raw files
 
+`mfma_calibration` (the matrix-core rate kernel, what an MFMA-bound kernel is compared with
+beside the published peak) is collected and summarised like a workload when named: kernel
+trace, the instruction counters and the clock, per instruction mix.
+
 `collect` runs, per workload, one `rocprofv3 --kernel-trace --stats` pass and one `--pmc`
 pass per counter group (every pass is its own process: rocprofv3 does not split counters
 over passes, and a group holds at most 8 SQ counters), always with `python3 bench.py ...`
@@ -48,12 +52,26 @@ COPY_BYTES = 2 * 65536 * 8 * 128 * 2  # read (and written) by one launch of copy
 XCDS = 8  # GRBM counters are summed over the part's 8 XCDs
 
 
+CAL = "mfma_calibration"
+CAL_GROUPS = [
+    ("sq1", "SQ_WAVES SQ_BUSY_CU_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_MFMA SQ_INSTS_SALU "
+            "SQ_INSTS_LDS SQ_INSTS_VALU_TRANS_F32"),
+    ("grbm", "GRBM_GUI_ACTIVE"),
+]
+
+
 def trace_cmd(w: str, out: Path) -> list[str]:
+    if w == CAL:
+        return ["rocprofv3", "--kernel-trace", "--stats", "-d", str(out / "trace"), "-o", "t", "--output-format",
+                "csv", "--", "python3", "bench.py", "--workload", w, "--steps", "2", "--no-cpu"]
     return ["rocprofv3", "--kernel-trace", "--stats", "-d", str(out / "trace"), "-o", "t", "--output-format",
             "csv", "--", "python3", "bench.py", "--workload", w, "--steps", "20", "--warmup", "3", "--no-cpu"]
 
 
 def pmc_cmd(w: str, out: Path, tag: str, counters: str) -> list[str]:
+    if w == CAL:
+        return ["rocprofv3", "--pmc", *counters.split(), "-d", str(out / tag), "-o", "p", "--output-format", "csv",
+                "--", "python3", "bench.py", "--workload", w, "--steps", "1", "--no-cpu"]
     return ["rocprofv3", "--pmc", *counters.split(), "-d", str(out / tag), "-o", "p", "--output-format", "csv",
             "--", "python3", "bench.py", "--workload", w, "--steps", "5", "--warmup", "2", "--no-cpu",
             "--ramp-ms", "0"]
@@ -70,7 +88,7 @@ def collect(workloads: list[str]) -> int:
         out = RAW / w
         subprocess.run(["rm", "-rf", str(out)], check=True)
         out.mkdir(parents=True)
-        groups = TRAFFIC_GROUPS + (SQ_GROUPS if w in MFMA_BOUND else [])
+        groups = CAL_GROUPS if w == CAL else TRAFFIC_GROUPS + (SQ_GROUPS if w in MFMA_BOUND else [])
         cmds = [("trace", trace_cmd(w, out))] + [(tag, pmc_cmd(w, out, tag, c)) for tag, c in groups]
         for tag, cmd in cmds:
             print(f"== {w} / {tag}", flush=True)
@@ -89,7 +107,7 @@ def collect(workloads: list[str]) -> int:
 
 
 def short(name: str) -> str:
-    return name.replace("ghip::(anonymous namespace)::", "").replace("ghip::", "").replace("void ", "").split("(")[0]
+    return (name.replace("(anonymous namespace)::", "").replace("ghip::", "").replace("void ", "")).split("(")[0]
 
 
 def counters(w: str, tag: str) -> dict:
@@ -162,8 +180,98 @@ def calibration():
     return COPY_BYTES / 1024 / fk, COPY_BYTES / 1024 / wk, fk, wk
 
 
+def cal_kernel(name: str):
+    """(wide shape?, fma, exp, lds, salu per pair of MFMAs) from `mfma_rate_kernel<true, 6, 2, 3, 4>`."""
+    args = name[name.index("<") + 1:name.rindex(">")].split(",")
+    return args[0].strip() == "true", tuple(int(a) for a in args[1:5])
+
+
+def summarise_calibration() -> None:
+    """profiles/mfma_calibration.md: per instruction mix the kernel-trace duration (the timed
+    launches: the longest grid of 512-thread or 256-thread workgroups), the TFLOP/s that
+    follows from it, the instructions a wave issues per MFMA (counters) and the clock."""
+    out = RAW / CAL
+    res = bench_line(CAL)["workloads"][CAL]
+    flops_per_wave = 20000 * 16 * 2.0 * 32 * 32 * 16
+    trace = collections.defaultdict(list)  # (kernel, workgroup size) -> durations
+    for f in glob.glob(str(out / "trace" / "**" / "*kernel_trace.csv"), recursive=True):
+        for r in csv.DictReader(open(f)):
+            k = short(r["Kernel_Name"])
+            if k.startswith("mfma_rate_kernel"):
+                trace[(k, int(r["Workgroup_Size_X"]))].append(float(r["End_Timestamp"]) - float(r["Start_Timestamp"]))
+    cnt = collections.defaultdict(lambda: collections.defaultdict(list))
+    clock = collections.defaultdict(list)
+    for tag, _ in CAL_GROUPS:
+        for f in glob.glob(str(out / tag / "**" / "*counter_collection.csv"), recursive=True):
+            for r in csv.DictReader(open(f)):
+                k = short(r["Kernel_Name"])
+                if not k.startswith("mfma_rate_kernel"):
+                    continue
+                key = (k, int(r["Workgroup_Size"]) if "Workgroup_Size" in r else int(r["Workgroup_Size_X"]))
+                cnt[key][r["Counter_Name"]].append(float(r["Counter_Value"]))
+                if r["Counter_Name"] == "GRBM_GUI_ACTIVE":
+                    ns = float(r["End_Timestamp"]) - float(r["Start_Timestamp"])
+                    if ns > 0:
+                        clock[key].append(float(r["Counter_Value"]) / XCDS / ns)
+    L = [f"# {CAL}: what the matrix cores reach, by instruction mix ({res['workload']})", "",
+         "Commands (from the repository root on one MI355X, `export TMPDIR=/tmp` first; OUT is any scratch folder):",
+         "", "```", shown(trace_cmd(CAL, out))]
+    L += [shown(pmc_cmd(CAL, out, tag, c)) for tag, c in CAL_GROUPS] + ["```", ""]
+    L += ["`mfma_rate_kernel<wide, fma, exp, lds, salu>` of `libgranite_hip_calibration.so`: one workgroup per "
+          "compute unit, one (256 threads) or two (512) waves per SIMD, 20000 passes of 16 `v_mfma_f32_32x32x16_f16` "
+          "per wave on register operands (normally distributed fp16 unless said otherwise), and per pair of MFMAs "
+          "`fma` float FMAs, `exp` `v_exp_f32`, `lds` 16-byte LDS reads whose data feeds later MFMAs and `salu` "
+          "scalar additions.  Every launch is preceded by three untimed ones; durations are the kernel trace's, "
+          "the best launch per mix.  TFLOP/s counts MFMA flops only; the published peak is 2500.", "",
+          "| mix per MFMA | waves per SIMD | best ns | TFLOP/s | of 2500 | VALU per MFMA | of them exp | LDS per MFMA | "
+          "SALU per MFMA | MFMA busy | clock GHz |", "|---|---|---|---|---|---|---|---|---|---|---|"]
+    rows = {}
+    for (k, wg), durs in sorted(trace.items()):
+        wide, mix = cal_kernel(k)
+        if not wide:
+            continue
+        best = min(durs)
+        waves = wg // 256
+        tf = 256 * 4 * waves * flops_per_wave / (best * 1e-9) / 1e12
+        c = {n: mean(v) for n, v in cnt.get((k, wg), {}).items()}
+        per = lambda n: (c[n] / c["SQ_INSTS_MFMA"]) if c.get("SQ_INSTS_MFMA") else float("nan")
+        valu = per("SQ_INSTS_VALU") - 1 if c.get("SQ_INSTS_VALU") else float("nan")  # the counter includes the MFMAs
+        busy = (c["SQ_VALU_MFMA_BUSY_CYCLES"] / (4 * c["SQ_BUSY_CU_CYCLES"])) if c.get("SQ_BUSY_CU_CYCLES") else float("nan")
+        ghz = mean(clock[(k, wg)]) if clock.get((k, wg)) else float("nan")
+        label = (f"{mix[0] / 2:g} fma, {mix[1] / 2:g} exp, {mix[2] / 2:g} lds, {mix[3] / 2:g} salu" if any(mix) else "none")
+        rows[(mix, waves)] = tf
+        L.append(f"| {label} | {waves} | {best:.0f} | {tf:.0f} | {tf / 2500:.3f} | {valu:.2f} | "
+                 f"{per('SQ_INSTS_VALU_TRANS_F32'):.2f} | {per('SQ_INSTS_LDS'):.2f} | {per('SQ_INSTS_SALU'):.2f} | "
+                 f"{busy:.3f} | {ghz:.2f} |")
+    L += ["", "(All-zero operands and the 16x16x32 shape run in the same command; bench.py's own HIP-event figures "
+          f"of this run: `{json.dumps(res['rates_TFLOPs'])}`.)"]
+    # the prefill kernels against the rows that carry their instruction mix
+    notes = []
+    for w, mix, kernel in (("chunked_prefill", (6, 2, 3, 4), "attention_tiles_dma_kernel"),):
+        md = PROFILES / f"{w}.md"
+        if md.exists() and (mix, 2) in rows:
+            for line in md.read_text().splitlines():
+                if line.startswith("Roofline from the event timing:"):
+                    ach = json.loads(line[line.index("`") + 1:line.rindex("`")])["achieved"]
+                    notes.append(f"`{kernel}` on {w}: {ach:.0f} TFLOP/s by `profiles/{w}.md` = "
+                                 f"**{ach / rows[(mix, 2)]:.2f}** of the {rows[(mix, 2)]:.0f} TFLOP/s of the row that "
+                                 f"carries its instruction mix ({mix[0] / 2:g} fma, {mix[1] / 2:g} exp, {mix[2] / 2:g} lds, "
+                                 f"{mix[3] / 2:g} salu per MFMA, two waves per SIMD), and {ach / 2500:.3f} of the published "
+                                 f"peak.  (Different boxes differ by several per cent; both files should come from one "
+                                 f"`collect` call.)")
+    if notes:
+        L += ["", "## The prefill kernel against its own mix", ""] + notes
+    (PROFILES / f"{CAL}.md").write_text("\n".join(L) + "\n")
+    print(f"wrote profiles/{CAL}.md", flush=True)
+
+
 def summarise(workloads: list[str]) -> int:
     PROFILES.mkdir(exist_ok=True)
+    if CAL in workloads:
+        workloads = [w for w in workloads if w != CAL]
+        cal_last = True
+    else:
+        cal_last = False
     fetch_kib, write_kib, fetch_raw, write_raw = calibration()
     traffic_path = PROFILES / "traffic.json"
     traffic = json.loads(traffic_path.read_text()) if traffic_path.exists() else {}
@@ -243,6 +351,8 @@ def summarise(workloads: list[str]) -> int:
         (PROFILES / f"{w}.md").write_text("\n".join(L) + "\n")
         print(f"wrote profiles/{w}.md", flush=True)
     traffic_path.write_text(json.dumps(traffic, indent=2) + "\n")
+    if cal_last:
+        summarise_calibration()  # after the workloads: it quotes profiles/chunked_prefill.md
     return 0
 
 
@@ -250,7 +360,7 @@ def main() -> int:
     if len(sys.argv) < 2 or sys.argv[1] not in ("collect", "summarise"):
         print(__doc__)
         return 2
-    names = sys.argv[2:] or WORKLOADS
+    names = sys.argv[2:] or WORKLOADS + [CAL]
     if sys.argv[1] == "collect":
         if "copy_calibration" not in names:
             names = names + ["copy_calibration"]
