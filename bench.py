@@ -438,9 +438,10 @@ def bench_mfma_calibration(gpu, steps, warmup, cpu):
     mixes = {"mfma_only": (0, 0, 0, 0), "4_fma": (8, 0, 0, 0), "8_fma": (16, 0, 0, 0), "1_exp": (0, 2, 0, 0),
              "3_fma_1_exp": (6, 2, 0, 0), "1_lds_read": (0, 0, 2, 0), "3_fma_1_exp_1_lds_read": (6, 2, 2, 0),
              "3_fma_1_exp_half_lds_read": (6, 2, 1, 0),
+             "3_fma_1_exp_1.5_lds_reads": (6, 2, 3, 0),
              "tiles_dma_kernel_mix_3_fma_1_exp_1.5_lds_2_salu": (6, 2, 3, 4),
              "tiles_kernel_mix_4_fma_1_exp_1.5_lds_3_salu": (8, 2, 3, 6),
-             "rows64_mix_3.5_fma_1_exp_0.5_lds_1.5_salu": (7, 2, 1, 3)}
+             "rows64_mix_3.5_fma_1_exp_0.5_lds_1_salu": (7, 2, 1, 2)}
     mix_rates = {name: {f"{w}_wave_per_simd": rate("normal", 32, w, mix) for w in (1, 2)}
                  for name, mix in mixes.items()}
     return {"workload": "mfma_calibration_register_operands_one_workgroup_per_cu", "metric": "mfma_TFLOPs",

@@ -21,6 +21,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 constexpr int kWave = 64;
 constexpr uint32_t kLdsHalves = 16384;          // 32 KiB of operands in LDS for the mix form
@@ -35,7 +36,9 @@ constexpr size_t kLdsBytes = 100 * 1024;        // and enough LDS to keep one wo
 // kWide: 32x32x16 (16 MFMAs a pass) or 16x16x32 (32 MFMAs a pass, the same flops).
 // kFma, kExp, kLds, kSalu: instructions per PAIR of MFMAs; the first MFMA of a pair is followed
 // by the larger half of each.
-template <bool kWide, int kFma, int kExp, int kLds, int kSalu>
+// kZeros only names the instantiation (all-zero operands), so that a kernel trace tells the two
+// kinds of run apart; the code is the same.
+template <bool kWide, int kFma, int kExp, int kLds, int kSalu, bool kZeros>
 __global__ void __launch_bounds__(512, 1)
     mfma_rate_kernel(const uint4v* __restrict__ operands, uint32_t n_vec, uint32_t iterations,
                      float* sink) {
@@ -72,23 +75,34 @@ __global__ void __launch_bounds__(512, 1)
         uint4v ld[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) ld[i] = __builtin_bit_cast(uint4v, a[i]);
-        const uint4v* lp = s_operands + lane;  // 64 lanes x 16 bytes: every bank once
+        // LDS operands: an odd count per pair makes the second MFMA's operand two 8-byte reads
+        // (as a V^T operand is), the first one's a 16-byte read (as a K operand is); every byte
+        // read feeds an MFMA.  Offsets are immediates; the base is re-declared every pass so
+        // that the reads stay in the loop.
+        uint32_t lds_base = lane * 16;  // 64 lanes x 16 bytes: every bank once
+        const unsigned char* const lds_bytes = reinterpret_cast<const unsigned char*>(s_operands);
         uint32_t scalar = iterations;
         for (uint32_t it = 0; it < iterations; it++) {
+            asm volatile("" : "+v"(lds_base));
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const bool second = r & 1;  // of the pair
                 const half8 aa = kLds > 0 ? __builtin_bit_cast(half8, ld[r & 3]) : a[r & 3];
                 c[r & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aa, b[(r + (r >> 2)) & 3], c[r & 3], 0, 0, 0);
-#pragma unroll
-                for (int j = 0; j < (second ? kLds / 2 : (kLds + 1) / 2); j++)
-                    ld[(r + 2 + j) & 3] = lp[64 * ((r + j + it) & 15)];  // used two MFMAs on
+                const int reads = second ? kLds / 2 : (kLds + 1) / 2;  // issued now, used two MFMAs on
+                if (reads == 1) {
+                    ld[(r + 2) & 3] = *reinterpret_cast<const uint4v*>(lds_bytes + lds_base + 1024 * (r & 15));
+                } else if (reads == 2) {
+                    const uint2v lo = *reinterpret_cast<const uint2v*>(lds_bytes + lds_base + 1024 * (r & 15));
+                    const uint2v hi = *reinterpret_cast<const uint2v*>(lds_bytes + lds_base + 1024 * ((r + 5) & 15) + 8);
+                    ld[(r + 2) & 3] = uint4v{lo.x, lo.y, hi.x, hi.y};
+                }
 #pragma unroll
                 for (int j = 0; j < (second ? kFma / 2 : (kFma + 1) / 2); j++)
                     x[(r + j) & 7] = __builtin_fmaf(x[(r + j) & 7], 0.999f, 0.001f);
 #pragma unroll
                 for (int j = 0; j < (second ? kExp / 2 : (kExp + 1) / 2); j++)
-                    e[(r + j) & 3] = __builtin_amdgcn_exp2f(e[(r + j) & 3] * 0.5f);
+                    e[(r + j) & 3] = __builtin_amdgcn_exp2f(-e[(r + j) & 3]);  // stays in [0.5, 1]
 #pragma unroll
                 for (int j = 0; j < (second ? kSalu / 2 : (kSalu + 1) / 2); j++)
                     asm volatile("s_add_u32 %0, %0, 3" : "+s"(scalar));
@@ -121,10 +135,10 @@ __global__ void __launch_bounds__(512, 1)
     if (total == 1.2345e-30f) sink[0] = total;  // keeps the loop alive; practically never taken
 }
 
-template <bool kWide, int kFma, int kExp, int kLds, int kSalu>
+template <bool kWide, int kFma, int kExp, int kLds, int kSalu, bool kZeros = false>
 int run(const uint4v* operands, uint32_t n_vec, uint32_t iterations, uint32_t workgroups, uint32_t threads,
         float* sink, float* milliseconds) {
-    auto kernel = mfma_rate_kernel<kWide, kFma, kExp, kLds, kSalu>;
+    auto kernel = mfma_rate_kernel<kWide, kFma, kExp, kLds, kSalu, kZeros>;
     CAL_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes)));
     hipEvent_t start, stop;
@@ -162,11 +176,23 @@ extern "C" int granite_hip_cal_mfma_mix(int device, const void* operands_f16, ui
     const auto* ops = static_cast<const uint4v*>(operands_f16);
     const uint32_t n_vec = uint32_t(n_halves / 8);
     const int mix = fma_per_pair * 1000 + exp_per_pair * 100 + lds_reads_per_pair * 10 + salu_per_pair;
+    // all-zero operands get an instantiation of their own (same code, another name in a trace)
+    bool zeros = true;
+    {
+        uint32_t head[1024];
+        CAL_CHECK(hipMemcpy(head, operands_f16, sizeof(head), hipMemcpyDeviceToHost));
+        for (uint32_t w : head) zeros = zeros && w == 0;
+    }
     int rc = -1;
 #define GHIP_CAL_MIX(f, e, l, sa)                                                                          \
     if (shape == 32 && mix == (f) * 1000 + (e) * 100 + (l) * 10 + (sa))                                    \
         rc = run<true, f, e, l, sa>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
-    if (shape == 16 && mix == 0) rc = run<false, 0, 0, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
+    if (shape == 16 && mix == 0)
+        rc = zeros ? run<false, 0, 0, 0, 0, true>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds)
+                   : run<false, 0, 0, 0, 0>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
+    if (shape == 32 && mix == 0 && zeros)
+        rc = run<true, 0, 0, 0, 0, true>(ops, n_vec, iterations, workgroups, threads, sink, milliseconds);
+    else
     GHIP_CAL_MIX(0, 0, 0, 0)
     GHIP_CAL_MIX(8, 0, 0, 0)   // 4 float FMAs per MFMA
     GHIP_CAL_MIX(16, 0, 0, 0)  // 8
@@ -175,9 +201,10 @@ extern "C" int granite_hip_cal_mfma_mix(int device, const void* operands_f16, ui
     GHIP_CAL_MIX(0, 0, 2, 0)   // 1 LDS read
     GHIP_CAL_MIX(6, 2, 2, 0)   // 3 FMAs + 1 exponential + 1 LDS read
     GHIP_CAL_MIX(6, 2, 1, 0)   // ... + half an LDS read (an operand feeding two MFMAs)
+    GHIP_CAL_MIX(6, 2, 3, 0)   // 3 FMAs + 1 exponential + 1.5 LDS reads (a K operand, a V^T operand as two)
     GHIP_CAL_MIX(6, 2, 3, 4)   // what attention_tiles_dma_kernel issues: 3 + 1 vector, 1.5 LDS, 2 scalar
     GHIP_CAL_MIX(8, 2, 3, 6)   // what attention_tiles_kernel issues: 4 + 1 vector, 1.5 LDS, 3 scalar
-    GHIP_CAL_MIX(7, 2, 1, 3)   // a 64-rows-per-wave form of the former: 3.5 + 1 vector, 0.5 LDS, 1.5 scalar
+    GHIP_CAL_MIX(7, 2, 1, 2)   // a 64-rows-per-wave form: 3.5 + 1 vector, 0.5 LDS, 1 scalar
 #undef GHIP_CAL_MIX
     (void)hipFree(sink);
     // 16 MFMAs of 2 * 32 * 32 * 16 flops (or 32 of half that) per pass and wave

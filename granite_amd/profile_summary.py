@@ -181,9 +181,10 @@ def calibration():
 
 
 def cal_kernel(name: str):
-    """(wide shape?, fma, exp, lds, salu per pair of MFMAs) from `mfma_rate_kernel<true, 6, 2, 3, 4>`."""
-    args = name[name.index("<") + 1:name.rindex(">")].split(",")
-    return args[0].strip() == "true", tuple(int(a) for a in args[1:5])
+    """(wide shape?, (fma, exp, lds, salu) per pair of MFMAs, zero operands?) from
+    `mfma_rate_kernel<true, 6, 2, 3, 0, false>`."""
+    args = [a.strip() for a in name[name.index("<") + 1:name.rindex(">")].split(",")]
+    return args[0] == "true", tuple(int(a) for a in args[1:5]), args[5] == "true"
 
 
 def summarise_calibration() -> None:
@@ -220,14 +221,14 @@ def summarise_calibration() -> None:
     L += ["`mfma_rate_kernel<wide, fma, exp, lds, salu>` of `libgranite_hip_calibration.so`: one workgroup per "
           "compute unit, one (256 threads) or two (512) waves per SIMD, 20000 passes of 16 `v_mfma_f32_32x32x16_f16` "
           "per wave on register operands (normally distributed fp16 unless said otherwise), and per pair of MFMAs "
-          "`fma` float FMAs, `exp` `v_exp_f32`, `lds` 16-byte LDS reads whose data feeds later MFMAs and `salu` "
+          "`fma` float FMAs, `exp` `v_exp_f32`, `lds` LDS operand reads whose data feeds later MFMAs and `salu` "
           "scalar additions.  Every launch is preceded by three untimed ones; durations are the kernel trace's, "
           "the best launch per mix.  TFLOP/s counts MFMA flops only; the published peak is 2500.", "",
           "| mix per MFMA | waves per SIMD | best ns | TFLOP/s | of 2500 | VALU per MFMA | of them exp | LDS per MFMA | "
           "SALU per MFMA | MFMA busy | clock GHz |", "|---|---|---|---|---|---|---|---|---|---|---|"]
     rows = {}
     for (k, wg), durs in sorted(trace.items()):
-        wide, mix = cal_kernel(k)
+        wide, mix, zeros = cal_kernel(k)
         if not wide:
             continue
         best = min(durs)
@@ -239,7 +240,10 @@ def summarise_calibration() -> None:
         busy = (c["SQ_VALU_MFMA_BUSY_CYCLES"] / (4 * c["SQ_BUSY_CU_CYCLES"])) if c.get("SQ_BUSY_CU_CYCLES") else float("nan")
         ghz = mean(clock[(k, wg)]) if clock.get((k, wg)) else float("nan")
         label = (f"{mix[0] / 2:g} fma, {mix[1] / 2:g} exp, {mix[2] / 2:g} lds, {mix[3] / 2:g} salu" if any(mix) else "none")
-        rows[(mix, waves)] = tf
+        if zeros:
+            label += " (all-zero operands)"
+        else:
+            rows[(mix, waves)] = tf
         L.append(f"| {label} | {waves} | {best:.0f} | {tf:.0f} | {tf / 2500:.3f} | {valu:.2f} | "
                  f"{per('SQ_INSTS_VALU_TRANS_F32'):.2f} | {per('SQ_INSTS_LDS'):.2f} | {per('SQ_INSTS_SALU'):.2f} | "
                  f"{busy:.3f} | {ghz:.2f} |")

@@ -37,12 +37,15 @@ int granite_hip_cal_mfma_rate(int device, const void *operands_f16, uint64_t n_h
 /* The same with the mix given per PAIR of MFMAs (so that half an instruction per MFMA can be
  * asked for: an LDS operand that feeds two MFMAs) and with scalar instructions in it:
  * after every pair a wave issues fma_per_pair float FMAs, exp_per_pair v_exp_f32,
- * lds_reads_per_pair 16-byte LDS reads and salu_per_pair scalar additions, the larger half
- * of each after the first MFMA of the pair.  Supported (fma, exp, lds, salu), shape 32:
- * (0,0,0,0) (8,0,0,0) (16,0,0,0) (0,2,0,0) (6,2,0,0) (0,0,2,0) (6,2,2,0) (6,2,1,0) and the mixes
- * that the hardware counters report for the two prefill kernels, (6,2,3,4) for
- * attention_tiles_dma_kernel and (8,2,3,6) for attention_tiles_kernel, and (7,2,1,3), a
- * 64-rows-per-wave form; shape 16 with (0,0,0,0).  Everything else as above. */
+ * lds_reads_per_pair LDS operand reads and salu_per_pair scalar additions, the larger half
+ * of each after the first MFMA of the pair (an MFMA with two reads gets its operand as two
+ * 8-byte reads, as a V^T operand is read; with one as a 16-byte read).  Supported
+ * (fma, exp, lds, salu), shape 32: (0,0,0,0) (8,0,0,0) (16,0,0,0) (0,2,0,0) (6,2,0,0) (0,0,2,0)
+ * (6,2,2,0) (6,2,1,0) (6,2,3,0) and the mixes that the hardware counters report for the two
+ * prefill kernels, (6,2,3,4) for attention_tiles_dma_kernel and (8,2,3,6) for
+ * attention_tiles_kernel, and (7,2,1,2), a 64-rows-per-wave form; shape 16 with (0,0,0,0).  All-zero operands run an
+ * instantiation of their own, so that a kernel trace tells them apart.  Everything else as
+ * above. */
 int granite_hip_cal_mfma_mix(int device, const void *operands_f16, uint64_t n_halves,
                              uint32_t iterations, int shape, int waves_per_simd,
                              int fma_per_pair, int exp_per_pair, int lds_reads_per_pair,
