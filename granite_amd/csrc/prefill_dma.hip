@@ -100,23 +100,6 @@ __device__ __forceinline__ void dma_lanes(uint32_t lds_addr, const void* addr) {
                  :
                  : "s"(lds_addr), "v"(addr));
 }
-// An MFMA of the second product with the output block tied to its registers: left to
-// itself the compiler now and then moves the block to other registers through the MFMA
-// (destination != accumulator input), and the second home costs 64 registers where they
-// are scarcest.  Nothing reads an output block with a vector instruction inside the loop
-// except the rare rescale, which waits first (mfma_drain).
-__device__ __forceinline__ void mfma_output(float16v& o, const uint4v& a, const half8& b) {
-#ifdef GHIP_DMA_TIED_OUTPUT
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(o) : "v"(a), "v"(b));
-#else
-    o = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(a), b, o, 0, 0, 0);
-#endif
-}
-__device__ __forceinline__ void mfma_drain() {
-#ifdef GHIP_DMA_TIED_OUTPUT
-    asm volatile("s_nop 15\n\ts_nop 15");
-#endif
-}
 template <int kCount>
 __device__ __forceinline__ void wait_transfers() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCount));
@@ -340,7 +323,6 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     };
     // moves the reference of row block rb up to cover the scores `sacc`; rescales l and O
     auto rebase = [&](int rb, const float16v& sacc) __attribute__((always_inline)) {
-        mfma_drain();
         float mraw = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; r++) mraw = fmaxf(mraw, sacc[r]);
@@ -378,9 +360,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     auto accumulate = [&](uint32_t buf, uint32_t sub, const half8 (&bp)[kRB][2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 2 * kBlocks; i++) {
-            const uint4v a = v_pair(s_raw + vt_lane[i % kBlocks] + buf * kVTile + sub * 32 * 256 + (i / kBlocks) * 16 * 256);
+            const half8 a = as_half8(v_pair(s_raw + vt_lane[i % kBlocks] + buf * kVTile + sub * 32 * 256 + (i / kBlocks) * 16 * 256));
 #pragma unroll
-            for (int rb = 0; rb < kRB; rb++) mfma_output(oacc[rb][i % kBlocks], a, bp[rb][i / kBlocks]);
+            for (int rb = 0; rb < kRB; rb++)
+                oacc[rb][i % kBlocks] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp[rb][i / kBlocks], oacc[rb][i % kBlocks], 0, 0, 0);
         }
     };
 
@@ -397,10 +380,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     auto fused_phase = [&](auto kb, auto sub_q, auto vb, auto sub_v, bool masked, bool softmax_live, uint32_t j_q,
                            float16v (&s_out)[kRB], const float16v (&s_in)[kRB], half8 (&p_out)[kRB][2],
                            const half8 (&p_prev)[kRB][2], auto&& side) __attribute__((always_inline)) {
-#ifndef GHIP_DMA_RING
-#define GHIP_DMA_RING 3
-#endif
-        constexpr int kRing = GHIP_DMA_RING;
+        constexpr int kRing = 3;  // LDS operands are requested two MFMAs ahead
         uint4v ring[kRing];
 #pragma unroll
         for (int i = 0; i < kRing - 1; i++) ring[i] = k_operand(kb, sub_q, i);
@@ -446,7 +426,8 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             if (i + kRing - 1 < 2 * kBlocks) ring[(i + kRing - 1) % kRing] = v_operand(vb, sub_v, i + kRing - 1);
 #pragma unroll
             for (int rb = 0; rb < kRB; rb++) {
-                mfma_output(oacc[rb][i % kBlocks], ring[i % kRing], p_prev[rb][i / kBlocks]);
+                oacc[rb][i % kBlocks] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                    as_half8(ring[i % kRing]), p_prev[rb][i / kBlocks], oacc[rb][i % kBlocks], 0, 0, 0);
                 softmax_step(rb, kSteps + i);
                 side(kRB * (kSteps + i) + rb);
                 __builtin_amdgcn_sched_barrier(0);
@@ -529,6 +510,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         }
         // This iteration's transfers: K of tile it + 3 and V of tile it + 2 into buffers kbuf, vbuf.
         const auto stage_next = [&](uint32_t it, uint32_t kbuf, uint32_t vbuf, int piece) __attribute__((always_inline)) {
+
             if (piece == 0 && it + 2 < n_tiles) stage_v(it + 2, vbuf, v_row);
             if (piece == 1 && it + 3 < n_tiles) {
                 const uint32_t row = group_row(it + 3, entry_next);
@@ -554,12 +536,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             const uint32_t j = 2 * it;
             fused_phase(IC<B>{}, IC<1>{}, IC<(B + 3) & 3>{}, IC<1>{}, j + 1 >= j_mask, j < j_end, j + 1, s1, s0,
                         p_new, p_old, [&](int slot) __attribute__((always_inline)) {
-#ifndef GHIP_DMA_SLOT_V
-#define GHIP_DMA_SLOT_V 9
-#define GHIP_DMA_SLOT_K 11
-#endif
-                            if (slot == GHIP_DMA_SLOT_V) stage_next(it, (B + 3) & 3, (B + 2) & 3, 0);
-                            if (slot == GHIP_DMA_SLOT_K) stage_next(it, (B + 3) & 3, (B + 2) & 3, 1);
+                            // (after the 10th and 12th MFMA of the first phase: measured best by 1 %)
+                            if (slot == 9) stage_next(it, (B + 3) & 3, (B + 2) & 3, 0);
+                            if (slot == 11) stage_next(it, (B + 3) & 3, (B + 2) & 3, 1);
                         });
             fused_phase(IC<(B + 1) & 3>{}, IC<0>{}, IC<B>{}, IC<0>{}, j + 2 >= j_mask, j + 1 < j_end, j + 2, s0, s1,
                         p_old, p_new, [](int) {});
@@ -593,7 +572,6 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
 
     if (!wave_active) return;
-    mfma_drain();
 #pragma unroll
     for (int rb = 0; rb < kRB; rb++) {
         const LanePair both = half_wave_pair(l_run[rb]);

@@ -13,6 +13,7 @@
 #include "granite/operators.h"
 #include "granite/paged_batch.h"
 #include "granite/rope.h"
+#include "granite/tree_verify.h"
 #include "granite_hip.h"
 #include "host_memory_backend.h"
 
@@ -589,6 +590,93 @@ TEST_CASE(paged_decode_batch_checks) {
     CHECK_CODE(step.initialize(&pool, 4, 4, &be), ErrorCode::BackendNotSupported);
     const int slots[1] = {0};
     CHECK_CODE(step.begin_step(std::span<const int>(slots, 1)), ErrorCode::InvalidState);
+}
+
+// The branch order of TransformerModel::attention_gpu (src/llm/transformer.mm:4837-5051).
+TEST_CASE(attention_gpu_dispatch_decision) {
+    AttentionRequest r;
+    r.total_tokens = 1;
+    r.start_pos = 40;
+    r.paged_attention = true;
+    r.has_gpu_cache = true;
+    r.gpu_cache_len = 12;      // paged attention wins whatever the contiguous GPU cache holds (:4850)
+    auto path = select_attention_path(r);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::PagedDecode);
+
+    r.paged_attention = false;
+    r.gpu_cache_max_seq_len = 4096;
+    r.gpu_cache_len = 40;      // in sync: the full GPU decode (:4878)
+    path = select_attention_path(r);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::FullDecode);
+
+    r.gpu_cache_len = 30;      // behind the host cache, which covers start_pos: sync, then decode (:4890)
+    r.host_cache_len = 40;
+    path = select_attention_path(r);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::SyncThenFullDecode);
+    r.host_cache_len = 35;     // the host cache does not cover it either: the reference goes to its CPU path
+    CHECK_CODE(select_attention_path(r), ErrorCode::InvalidState);
+    r.host_cache_len = -1;
+    r.gpu_cache_len = 50;      // ahead: "something is wrong" (:4911)
+    CHECK_CODE(select_attention_path(r), ErrorCode::InvalidState);
+
+    // the offload branch comes before the decode branches and leaves the GPU (:4861-4872)
+    r.kv_cache_offload = true;
+    r.gpu_cache_max_seq_len = 40;
+    r.gpu_cache_len = 40;
+    CHECK_CODE(select_attention_path(r), ErrorCode::BackendNotSupported);
+    r.gpu_cache_max_seq_len = 41;
+    path = select_attention_path(r);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::FullDecode);
+    r.paged_attention = true;  // ... but after the paged branch
+    r.gpu_cache_max_seq_len = 40;
+    path = select_attention_path(r);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::PagedDecode);
+
+    // several tokens: the GPU prefill only from position 0 and only with a GPU cache (:4915)
+    AttentionRequest p;
+    p.total_tokens = 300;
+    p.has_gpu_cache = true;
+    p.gpu_cache_max_seq_len = 4096;
+    path = select_attention_path(p);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::Prefill);
+    p.paged_attention = true;  // the paged branch is for single tokens only
+    path = select_attention_path(p);
+    REQUIRE(path.ok());
+    CHECK(path.value() == AttentionPath::Prefill);
+    p.start_pos = 64;
+    CHECK_CODE(select_attention_path(p), ErrorCode::InvalidState);
+    p.start_pos = 0;
+    p.has_gpu_cache = false;
+    CHECK_CODE(select_attention_path(p), ErrorCode::InvalidState);
+    p.total_tokens = 0;
+    CHECK_CODE(select_attention_path(p), ErrorCode::InvalidArgument);
+}
+
+TEST_CASE(tree_verify_checks) {
+    HostMemoryBackend be;
+    REQUIRE(be.initialize().ok());
+    TreeVerify verify;
+    const int parents[3] = {-1, 0, 0};
+    CHECK_CODE(verify.begin(parents), ErrorCode::InvalidState);
+    CHECK_CODE(verify.initialize(nullptr, 4, 8, &be), ErrorCode::InvalidState);
+    PagedKVConfig cfg;
+    cfg.block_size = 16;
+    cfg.num_blocks = 4;
+    cfg.num_layers = 1;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = 128;
+    BlockManager mgr;
+    REQUIRE(mgr.initialize(cfg, &be).ok());
+    PagedKVCache seq(&mgr);
+    CHECK_CODE(verify.initialize(&seq, 0, 8, &be), ErrorCode::InvalidArgument);
+    // never computed on a backend that is not the GPU
+    CHECK_CODE(verify.initialize(&seq, 4, 8, &be), ErrorCode::BackendNotSupported);
 }
 
 int main(int argc, char** argv) { return hosttest::run_all(argc, argv); }

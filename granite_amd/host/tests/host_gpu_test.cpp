@@ -13,6 +13,7 @@
 #include "granite/kv_cache.h"
 #include "granite/operators.h"
 #include "granite/paged_batch.h"
+#include "granite/tree_verify.h"
 #include "granite/rope.h"
 #include "granite_hip.h"
 
@@ -1043,6 +1044,165 @@ TEST_CASE(speculative_commit_of_accepted_path) {
     // an empty path only restores the length
     CHECK_OK(commit_tree_path(seq, original, std::span<const int>(), kt, vt, backend()));
     CHECK(seq.seq_len() == original);
+}
+
+// Tree verification as SpeculativeRunner::verify_tree drives it (src/llm/speculative_runner.cpp:
+// 586-674, 871-882) over a *paged* prefix: a prompt through ChunkedPrefill, a SpeculationTree
+// built with add_node, tree attention for two layers (TransformerModel::attention_tree_gpu,
+// src/llm/transformer.mm:2146-2402) against the oracle, the accepted path committed and the
+// surplus blocks freed, and then one batched decode step whose output must be the oracle's
+// on the committed sequence.
+TEST_CASE(tree_verify_commit_then_decode_over_paged_prefix) {
+    REQUIRE(backend() != nullptr);
+    ModelConfig cfg;
+    cfg.num_layers = 2;
+    cfg.num_heads = 8;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = D;
+    const int bs = 16, hq = 8, hkv = 2, max_blocks = 8, max_pos = max_blocks * bs, prompt = 45;
+    PagedKVPool pool;
+    REQUIRE(pool.initialize(cfg, 2, 12 * bs, bs, backend()).ok());
+    BlockManager& mgr = pool.block_manager();
+    RoPECache rope;
+    rope.initialize(max_pos, D, 10000.0f);
+    std::vector<float> cos_t(size_t(max_pos) * D / 2), sin_t(cos_t.size());
+    go_rope_table(cos_t.data(), sin_t.data(), max_pos, D, 10000.0f);
+    const float scale = 1.0f / std::sqrt(float(D));
+    const int slot = pool.acquire_slot();
+    REQUIRE(slot >= 0);
+    PagedKVCache& seq = pool.get_cache(slot);
+    uint32_t seed = 9100;
+
+    // ---- the prefix: a prompt of 45 tokens in chunks of 32 (its parity is checked elsewhere)
+    ChunkedPrefill prefill;
+    REQUIRE(prefill.initialize(&seq, max_blocks, backend()).ok());
+    prefill.set_rounding(GRANITE_HIP_ROUND_TRUNCATE);
+    REQUIRE(prefill.begin(prompt, 32).ok());
+    for (int l = 0; l < 2; ++l) {
+        Tensor Q = upload({prompt, hq, D}, DataType::FP32, randn(size_t(prompt) * hq * D, seed++));
+        Tensor K = upload({prompt, hkv, D}, DataType::FP32, randn(size_t(prompt) * hkv * D, seed++));
+        Tensor V = upload({prompt, hkv, D}, DataType::FP32, randn(size_t(prompt) * hkv * D, seed++));
+        Tensor O = Tensor::allocate({prompt, hq, D}, DataType::FP32, backend()).take();
+        CHECK_OK(prefill.run_layer(l, Q, K, V, O, scale, &rope));
+        (void)backend()->wait_for_completion();
+        for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+    }
+    prefill.finish();
+    REQUIRE(seq.seq_len() == prompt);
+    std::vector<std::vector<uint16_t>> want_k, want_v;  // the oracle's pools start from the device's bytes
+    for (int l = 0; l < 2; ++l) {
+        want_k.push_back(download<uint16_t>(mgr.k_cache(l)));
+        want_v.push_back(download<uint16_t>(mgr.v_cache(l)));
+    }
+
+    // ---- the tree: 11 nodes, two branches under the root, depth 4
+    SpeculationTree tree;
+    tree.add_node(100, -1);                       // 0
+    tree.add_node(101, 0); tree.add_node(102, 0); // 1 2
+    tree.add_node(103, 1); tree.add_node(104, 1); // 3 4
+    tree.add_node(105, 2);                        // 5
+    tree.add_node(106, 4); tree.add_node(107, 4); // 6 7
+    tree.add_node(108, 5);                        // 8
+    tree.add_node(109, 7); tree.add_node(110, 3); // 9 10
+    const std::vector<int> parents_int = tree.get_parent_indices();
+    std::vector<int32_t> parents(parents_int.begin(), parents_int.end());
+    const int N = int(tree.size());
+
+    TreeVerify verify;
+    CHECK_CODE(verify.begin(parents_int), ErrorCode::InvalidState);
+    REQUIRE(verify.initialize(&seq, max_blocks, 16, backend()).ok());
+    const int bad_parent[2] = {-1, 5};
+    CHECK_CODE(verify.begin(bad_parent), ErrorCode::InvalidArgument);
+    REQUIRE(verify.begin(parents_int).ok());
+    CHECK(verify.original_len() == prompt && verify.num_nodes() == N);
+    CHECK(seq.seq_len() == prompt);  // nothing is appended by the tree step
+    const int accepted_before_layers[1] = {0};
+    CHECK_CODE(verify.commit(accepted_before_layers), ErrorCode::InvalidState);
+
+    std::vector<int32_t> table(seq.block_table().begin(), seq.block_table().end());
+    std::vector<std::vector<uint16_t>> node_k, node_v;  // per layer [N, Hkv, D] halves (truncated)
+    for (int l = 0; l < 2; ++l) {
+        auto q = randn(size_t(N) * hq * D, seed++), k = randn(size_t(N) * hkv * D, seed++),
+             v = randn(size_t(N) * hkv * D, seed++);
+        Tensor Q = upload({N, hq, D}, DataType::FP32, q);
+        Tensor K = upload({N, hkv, D}, DataType::FP32, k);
+        Tensor V = upload({N, hkv, D}, DataType::FP32, v);
+        Tensor O = Tensor::allocate({N, hq, D}, DataType::FP32, backend()).take();
+        CHECK_OK(verify.run_layer(l, Q, K, V, O, scale));
+        // oracle: the tree's K/V as the cast leaves them (transformer.mm:2295-2304), floats [N, Hkv, D]
+        node_k.push_back(to_half(k));
+        node_v.push_back(to_half(v));
+        auto kf = to_float(node_k[l]), vf = to_float(node_v[l]);
+        std::vector<float> want(q.size());
+        CHECK(go_attention_tree(q.data(), want_k[l].data(), want_v[l].data(), table.data(), bs, 0, kf.data(),
+                                vf.data(), parents.data(), want.data(), nullptr, 1, N, hq, hkv, D, prompt,
+                                scale) == 0);
+        CHECK(close_enough(download<float>(O), want, "tree attention over the paged prefix"));
+        // the kept copy is [Hkv, N, D], bit for bit the truncated rows
+        auto kept = download<uint16_t>(verify.k_tree(l));
+        bool same = kept.size() == node_k[l].size();
+        for (int h = 0; h < hkv && same; ++h)
+            for (int n = 0; n < N && same; ++n)
+                for (int d = 0; d < D; ++d)
+                    same = same && kept[(size_t(h) * N + n) * D + d] == node_k[l][(size_t(n) * hkv + h) * D + d];
+        CHECK(same);
+        for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+    }
+
+    // ---- the target agrees with 100, 101, 104, 107 and then says 555 where the tree says 109
+    const std::vector<int32_t> target_choices = {100, 101, 104, 107, 555};
+    const std::vector<int> accepted = tree.find_accepted_nodes(target_choices);
+    REQUIRE((accepted == std::vector<int>{0, 1, 4, 7}));
+    const int free_before = mgr.num_free_blocks();
+    CHECK_OK(verify.commit(accepted));
+    const int committed = prompt + int(accepted.size());  // 49 tokens: 4 blocks
+    CHECK(seq.seq_len() == committed && seq.num_blocks() == 4);
+    CHECK(mgr.num_free_blocks() == free_before - 1);      // 45 tokens held 3 blocks
+    table.assign(seq.block_table().begin(), seq.block_table().end());
+    for (int l = 0; l < 2; ++l) {
+        for (size_t i = 0; i < accepted.size(); ++i) {
+            const int pos = prompt + int(i);
+            const size_t row = size_t(table[pos / bs]) * bs + pos % bs;
+            for (int h = 0; h < hkv; ++h)
+                for (int d = 0; d < D; ++d) {
+                    want_k[l][(row * hkv + h) * D + d] = node_k[l][(size_t(accepted[i]) * hkv + h) * D + d];
+                    want_v[l][(row * hkv + h) * D + d] = node_v[l][(size_t(accepted[i]) * hkv + h) * D + d];
+                }
+        }
+        CHECK(download<uint16_t>(mgr.k_cache(l)) == want_k[l]);  // bit exact, nothing else written
+        CHECK(download<uint16_t>(mgr.v_cache(l)) == want_v[l]);
+    }
+    CHECK_CODE(verify.commit(accepted), ErrorCode::InvalidState);  // one commit per begin()
+
+    // ---- the next decode step sees prompt + accepted path
+    PagedDecodeBatch step;
+    REQUIRE(step.initialize(&pool, 2, max_blocks, backend()).ok());
+    step.set_rounding(GRANITE_HIP_ROUND_TRUNCATE);
+    const int slots[1] = {slot};
+    auto failed = step.begin_step(slots);
+    REQUIRE(failed.ok() && failed.value().empty());
+    CHECK(seq.seq_len() == committed + 1);
+    std::vector<int32_t> tables(max_blocks, 0), seq_lens = {committed + 1};
+    std::copy(seq.block_table().begin(), seq.block_table().end(), tables.begin());
+    for (int l = 0; l < 2; ++l) {
+        auto q = randn(size_t(hq) * D, seed++), k = randn(size_t(hkv) * D, seed++), v = randn(size_t(hkv) * D, seed++);
+        Tensor Q = upload({1, hq, D}, DataType::FP32, q);
+        Tensor K = upload({1, hkv, D}, DataType::FP32, k);
+        Tensor V = upload({1, hkv, D}, DataType::FP32, v);
+        Tensor O = Tensor::allocate({1, hq, D}, DataType::FP32, backend()).take();
+        CHECK_OK(step.run_layer(l, Q, K, V, O, scale, &rope));
+        CHECK(go_rope_apply(q.data(), 1, hq, D, committed, cos_t.data(), sin_t.data(), max_pos) == 0);
+        CHECK(go_rope_apply(k.data(), 1, hkv, D, committed, cos_t.data(), sin_t.data(), max_pos) == 0);
+        go_paged_kv_cache_append_f32(want_k[l].data(), k.data(), tables.data(), hkv, D, committed, 1, bs);
+        go_paged_kv_cache_append_f32(want_v[l].data(), v.data(), tables.data(), hkv, D, committed, 1, bs);
+        std::vector<float> want(q.size());
+        go_batched_paged_decode(q.data(), want_k[l].data(), want_v[l].data(), tables.data(), seq_lens.data(),
+                                want.data(), nullptr, 1, hq, hkv, D, bs, max_blocks, scale);
+        CHECK(download<uint16_t>(mgr.k_cache(l)) == want_k[l]);
+        CHECK(download<uint16_t>(mgr.v_cache(l)) == want_v[l]);
+        CHECK(close_enough(download<float>(O), want, "decode step after the commit"));
+        for (Tensor* t : {&Q, &K, &V, &O}) backend()->destroy_buffer(t->buffer());
+    }
 }
 
 int main(int argc, char** argv) {
