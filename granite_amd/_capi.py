@@ -158,6 +158,7 @@ SIGNATURES = {
     "granite_hip_paged_kv_cache_append_ex": (
         _int, [_vp, _vp, _int, _i64, _i64, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _int, _u32]),
     "granite_hip_paged_kv_gather": (_int, [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32]),
+    "granite_hip_copy_rows": (_int, [_vp, C.c_int64, _vp, C.c_int64, C.c_uint64, _u32, _u32]),
     "granite_hip_multihead_attention": (
         _int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _f32, _u32]),
     "granite_hip_attention_tree": (

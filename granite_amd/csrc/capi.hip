@@ -562,6 +562,12 @@ int granite_hip_paged_kv_gather(void* dst_k, void* dst_v, const void* k_cache,
                                         head_dim, len, block_size, max_seq_len);
 }
 
+int granite_hip_copy_rows(void* dst, int64_t dst_row_bytes, const void* src, int64_t src_row_bytes,
+                          uint64_t rows, uint32_t copy_bytes, uint32_t fill_bytes) {
+    GHIP_REQUIRE_INIT();
+    return ghip::launch_copy_rows(dst, dst_row_bytes, src, src_row_bytes, rows, copy_bytes, fill_bytes);
+}
+
 // ---- projections on Q4_K weights ------------------------------------------------
 
 int granite_hip_fused_qkv_matvec_q4k_batched(const void* x, int64_t x_stride, const void* wq,

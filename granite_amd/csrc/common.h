@@ -103,6 +103,8 @@ int launch_kv_append_paged(const void* new_k, const void* new_v, int src_dtype,
 int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const void* v_cache,
                            const int32_t* block_table, uint32_t num_kv_heads, uint32_t head_dim,
                            uint32_t len, uint32_t block_size, uint32_t max_seq_len);
+int launch_copy_rows(void* dst, int64_t dst_row_bytes, const void* src, int64_t src_row_bytes, uint64_t rows,
+                     uint32_t copy_bytes, uint32_t fill_bytes);
 int launch_decode(const granite_hip_decode_args& a, const ScratchSource& scratch = {});
 int launch_attention(const granite_hip_attention_args& a, const ScratchSource& scratch = {});
 int launch_tree_mask(const int32_t* parents, uint32_t* mask_words, uint32_t num_nodes);

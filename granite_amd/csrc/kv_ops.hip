@@ -10,6 +10,8 @@
 // store (and one 16-byte or two 16-byte loads), consecutive threads cover a
 // row, so every 256-byte destination row is written by 16 adjacent lanes.
 // K and V go in one launch (blockIdx.y selects).
+#include <algorithm>
+
 #include "common.h"
 
 namespace ghip {
@@ -291,6 +293,38 @@ int launch_kv_gather_paged(void* dst_k, void* dst_v, const void* k_cache, const 
     {
         KernelTimerScope timer("kv_gather");
         kv_gather_kernel<<<dim3(blocks, 2), dim3(256), 0, ctx().stream>>>(p);
+    }
+    return launch_status();
+}
+
+// Rows of 2-byte elements copied between two pitches, the tail of every destination row filled
+// with zeros: pads [rows, d] to [rows, d_padded] (or slices the other way, with no fill).
+__global__ void __launch_bounds__(256) copy_rows_kernel(uint16_t* dst, int64_t dst_pitch, const uint16_t* src,
+                                                        int64_t src_pitch, uint64_t rows, uint32_t copy_elems,
+                                                        uint32_t fill_elems) {
+    const uint64_t total = rows * fill_elems;
+    for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += uint64_t(gridDim.x) * blockDim.x) {
+        const uint64_t r = i / fill_elems;
+        const uint32_t c = uint32_t(i - r * fill_elems);
+        dst[r * dst_pitch + c] = c < copy_elems ? src[r * src_pitch + c] : uint16_t(0);
+    }
+}
+
+int launch_copy_rows(void* dst, int64_t dst_row_bytes, const void* src, int64_t src_row_bytes, uint64_t rows,
+                     uint32_t copy_bytes, uint32_t fill_bytes) {
+    if (!dst || !src) return GRANITE_HIP_ENULL;
+    if (rows == 0 || fill_bytes == 0) return GRANITE_HIP_OK;
+    if (copy_bytes > fill_bytes || (copy_bytes | fill_bytes) % 2 || dst_row_bytes % 2 || src_row_bytes % 2 ||
+        dst_row_bytes < int64_t(fill_bytes) || src_row_bytes < int64_t(copy_bytes) ||
+        (reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 2)
+        return GRANITE_HIP_EINVAL;
+    const uint64_t work = rows * (fill_bytes / 2);
+    const uint32_t blocks = static_cast<uint32_t>(std::min<uint64_t>((work + 255) / 256, 65535u * 4));
+    {
+        KernelTimerScope timer("copy_rows");
+        copy_rows_kernel<<<dim3(blocks), dim3(256), 0, ctx().stream>>>(
+            static_cast<uint16_t*>(dst), dst_row_bytes / 2, static_cast<const uint16_t*>(src), src_row_bytes / 2, rows,
+            copy_bytes / 2, fill_bytes / 2);
     }
     return launch_status();
 }

@@ -5,7 +5,11 @@
 // shaped like Q, attributes `scale` (default 1/sqrt(D)) and `start_pos`
 // (default 0), key k visible to query q iff k <= q + start_pos
 // (metal_operators.mm:640-641).  Unlike that operator it works on the device
-// buffers in place (no map/copy round trip) and accepts head dimensions:
+// buffers in place (no map/copy round trip) and accepts head dimensions.  The
+// kernels exist for head sizes 64 and 128; any other size up to 128 is presented
+// to them zero-padded (zero columns add nothing to a score and give zero output
+// columns, which are sliced off again), so the reference's small test tensors
+// (head size 4, tests/test_vulkan.cpp:353-482) go through unchanged.  Shapes:
 //   Q, out  [seq_q, D] | [H, seq_q, D] | [B, H, seq_q, D]   FP16 or FP32
 //   K, V    [seq_kv, D] | [Hkv, seq_kv, D] | [B, Hkv, seq_kv, D]   FP16
 // with H a multiple of Hkv (grouped-query attention).  The extra attribute
@@ -64,8 +68,8 @@ class HipAttentionOp final : public IOperator {
             return Error(ErrorCode::DTypeMismatch, "K and V must be FP16 (the KV cache type)");
         if (!Q.is_contiguous() || !K.is_contiguous() || !V.is_contiguous())
             return Error(ErrorCode::InvalidArgument, "Q, K and V must be contiguous");
-        if (q.dim != 128 && q.dim != 64)
-            return Error(ErrorCode::NotImplemented, "HipAttentionOp has kernels for head_dim 64 and 128");
+        if (q.dim < 1 || q.dim > 128)
+            return Error(ErrorCode::NotImplemented, "HipAttentionOp serves head_dim 1 .. 128");
         return {};
     }
 
@@ -107,20 +111,56 @@ class HipAttentionOp final : public IOperator {
             return Error(ErrorCode::InvalidArgument, "Tensor buffers do not belong to the HIP backend");
 
         const int dtype = Q.dtype() == DataType::FP16 ? GRANITE_HIP_F16 : GRANITE_HIP_F32;
-        const size_t q_batch_bytes = size_t(q.heads * q.seq * q.dim) * dtype_size(Q.dtype());
-        const size_t kv_batch_bytes = size_t(k.heads * k.seq * k.dim) * sizeof(uint16_t);
+        const size_t q_esz = dtype_size(Q.dtype());
+        // head sizes without a kernel: zero-padded copies of Q, K and V, and a padded output
+        const int64_t dim = q.dim == 64 || q.dim == 128 ? q.dim : (q.dim < 64 ? 64 : 128);
+        const bool padded = dim != q.dim;
+        const uint64_t q_rows = uint64_t(q.batch * q.heads * q.seq), kv_rows = uint64_t(k.batch * k.heads * k.seq);
+        BufferHandle tmp[4] = {};  // Q, K, V, out
+        auto release = [&] {
+            for (BufferHandle& h : tmp)
+                if (h.valid()) ctx.backend->destroy_buffer(h);
+        };
+        if (padded) {
+            const size_t bytes[4] = {q_rows * dim * q_esz, kv_rows * dim * 2, kv_rows * dim * 2, q_rows * dim * q_esz};
+            char* const src[3] = {q_ptr, k_ptr, v_ptr};
+            const size_t esz[3] = {q_esz, 2, 2};
+            const uint64_t rows[3] = {q_rows, kv_rows, kv_rows};
+            Result<void> status;
+            for (int i = 0; i < 4 && status.ok(); ++i) {
+                auto made = ctx.backend->create_buffer(BufferDesc::device(bytes[i]));
+                if (!made.ok()) status = made.error();
+                else tmp[i] = made.value();
+            }
+            for (int i = 0; i < 3 && status.ok(); ++i)
+                status = hip_status_to_result(
+                    granite_hip_copy_rows(hip_device_pointer(ctx.backend, tmp[i]), int64_t(dim * esz[i]), src[i],
+                                          int64_t(q.dim * esz[i]), rows[i], uint32_t(q.dim * esz[i]),
+                                          uint32_t(dim * esz[i])),
+                    "granite_hip_copy_rows");
+            if (!status.ok()) {
+                release();
+                return status;
+            }
+            q_ptr = static_cast<char*>(hip_device_pointer(ctx.backend, tmp[0]));
+            k_ptr = static_cast<char*>(hip_device_pointer(ctx.backend, tmp[1]));
+            v_ptr = static_cast<char*>(hip_device_pointer(ctx.backend, tmp[2]));
+        }
+        char* const result_ptr = padded ? static_cast<char*>(hip_device_pointer(ctx.backend, tmp[3])) : o_ptr;
+        const size_t q_batch_bytes = size_t(q.heads * q.seq * dim) * q_esz;
+        const size_t kv_batch_bytes = size_t(k.heads * k.seq * dim) * sizeof(uint16_t);
 
         HipCompute compute;  // stateless façade over the already initialised library
         for (int64_t b = 0; b < q.batch; ++b) {
             granite_hip_attention_args a{};
             a.q = q_ptr + b * q_batch_bytes;
             a.q_dtype = dtype;
-            a.q_tok_stride = q.dim;
-            a.q_head_stride = q.seq * q.dim;
-            a.out = o_ptr + b * q_batch_bytes;
+            a.q_tok_stride = dim;
+            a.q_head_stride = q.seq * dim;
+            a.out = result_ptr + b * q_batch_bytes;
             a.out_dtype = dtype;
-            a.out_tok_stride = q.dim;
-            a.out_head_stride = q.seq * q.dim;
+            a.out_tok_stride = dim;
+            a.out_head_stride = q.seq * dim;
             a.k_cache = k_ptr + b * kv_batch_bytes;
             a.v_cache = v_ptr + b * kv_batch_bytes;
             a.max_seq = static_cast<uint32_t>(k.seq);
@@ -130,9 +170,21 @@ class HipAttentionOp final : public IOperator {
             a.seq_q = static_cast<uint32_t>(q.seq);
             a.num_heads = static_cast<uint32_t>(q.heads);
             a.num_kv_heads = static_cast<uint32_t>(k.heads);
-            a.head_dim = static_cast<uint32_t>(q.dim);
+            a.head_dim = static_cast<uint32_t>(dim);
             a.scale = static_cast<float>(scale);
-            GRANITE_TRY(compute.attention(a));
+            if (auto launched = compute.attention(a); !launched.ok()) {
+                release();
+                return launched;
+            }
+        }
+        if (padded) {
+            auto sliced = hip_status_to_result(
+                granite_hip_copy_rows(o_ptr, int64_t(q.dim * q_esz), result_ptr, int64_t(dim * q_esz), q_rows,
+                                      uint32_t(q.dim * q_esz), uint32_t(q.dim * q_esz)),
+                "granite_hip_copy_rows");
+            (void)ctx.backend->wait_for_completion();  // the temporaries are released below
+            release();
+            return sliced;
         }
         return {};
     }

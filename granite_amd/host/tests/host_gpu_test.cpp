@@ -181,21 +181,22 @@ TEST_CASE(backend_buffers) {
 
 // The reference's attention known-answer test (tests/test_vulkan.cpp:353-482):
 // Sq=2, Skv=3, D=4, no mask, Q[i]=i+1, K^T[i]=(i+1)/2, V[i]=(i+1)/4, scale 0.5,
-// tolerance 1e-4.  All inputs are exact in binary16.  The head dimension is
-// embedded in 128 columns of zeros, which changes neither scores nor the first
-// four output columns.  Expected values: tests/golden/vulkan_attention_kat.json.
+// tolerance 1e-4.  All inputs are exact in binary16.  The tensors go through the registry as
+// the reference shapes them ([2, 4] and [3, 4]); the operator pads head size 4 to 64 itself.
+// Expected values: tests/golden/vulkan_attention_kat.json.
 TEST_CASE(operator_known_answer) {
     REQUIRE(backend() != nullptr);
     const double expected[2][4] = {
         {2.162234681491403, 2.412234681491403, 2.662234681491403, 2.912234681491403},
         {2.248494307269034, 2.498494307269034, 2.748494307269034, 2.998494307269034}};
-    std::vector<float> q(2 * D, 0.0f), k(3 * D, 0.0f), v(3 * D, 0.0f);
+    // the reference's tensors as they are: Q [2, 4], K and V [3, 4]
+    std::vector<float> q(2 * 4), k(3 * 4), v(3 * 4);
     for (int i = 0; i < 2; ++i)
-        for (int d = 0; d < 4; ++d) q[i * D + d] = float(i * 4 + d + 1);
+        for (int d = 0; d < 4; ++d) q[i * 4 + d] = float(i * 4 + d + 1);
     for (int d = 0; d < 4; ++d)
-        for (int t = 0; t < 3; ++t) k[t * D + d] = float(d * 3 + t + 1) * 0.5f;  // K^T is [D, T]
+        for (int t = 0; t < 3; ++t) k[t * 4 + d] = float(d * 3 + t + 1) * 0.5f;  // K^T is [D, T]
     for (int t = 0; t < 3; ++t)
-        for (int d = 0; d < 4; ++d) v[t * D + d] = float(t * 4 + d + 1) * 0.25f;
+        for (int d = 0; d < 4; ++d) v[t * 4 + d] = float(t * 4 + d + 1) * 0.25f;
 
     initialize_operators();
     auto op = OperatorRegistry::instance().create(OpType::ScaledDotProductAttention,
@@ -204,11 +205,12 @@ TEST_CASE(operator_known_answer) {
     for (DataType qdt : {DataType::FP32, DataType::FP16}) {
         OpContext ctx;
         ctx.backend = backend();
-        Tensor Q = qdt == DataType::FP32 ? upload({2, D}, qdt, q) : upload({2, D}, qdt, to_half(q));
-        ctx.inputs = {Q, upload({3, D}, DataType::FP16, to_half(k)),
-                      upload({3, D}, DataType::FP16, to_half(v))};
+        Tensor Q = qdt == DataType::FP32 ? upload({2, 4}, qdt, q) : upload({2, 4}, qdt, to_half(q));
+        ctx.inputs = {Q, upload({3, 4}, DataType::FP16, to_half(k)),
+                      upload({3, 4}, DataType::FP16, to_half(v))};
         auto shapes = op->infer_shapes(ctx);
         REQUIRE(shapes.ok());
+        CHECK((shapes.value()[0] == std::vector<int64_t>{2, 4}));
         auto out = Tensor::allocate(shapes.value()[0], qdt, backend());
         REQUIRE(out.ok());
         ctx.outputs = {out.take()};
@@ -218,14 +220,58 @@ TEST_CASE(operator_known_answer) {
         CHECK_OK(op->execute(ctx));
         std::vector<float> got = qdt == DataType::FP32 ? download<float>(ctx.outputs[0])
                                                        : to_float(download<uint16_t>(ctx.outputs[0]));
+        REQUIRE(got.size() == 8);
         const double tol = qdt == DataType::FP32 ? 1e-4 : 2e-3;  // fp16 output rounding
-        for (int i = 0; i < 2; ++i) {
-            for (int d = 0; d < 4; ++d) CHECK(std::fabs(got[i * D + d] - expected[i][d]) <= tol);
-            for (int d = 4; d < D; ++d) CHECK(got[i * D + d] == 0.0f);
-        }
+        for (int i = 0; i < 2; ++i)
+            for (int d = 0; d < 4; ++d) CHECK(std::fabs(got[i * 4 + d] - expected[i][d]) <= tol);
         for (auto& t : ctx.inputs) backend()->destroy_buffer(t.buffer());
         backend()->destroy_buffer(ctx.outputs[0].buffer());
     }
+}
+
+// A head size with no kernel of its own (80, then 24 and 100): the operator pads to 128 or 64,
+// the result must be the oracle's for the unpadded tensors.  Causal, grouped-query, start_pos > 0.
+TEST_CASE(operator_other_head_sizes_vs_oracle) {
+    REQUIRE(backend() != nullptr);
+    initialize_operators();
+    auto op = OperatorRegistry::instance().create(OpType::ScaledDotProductAttention, BackendType::HIP);
+    REQUIRE(op != nullptr);
+    for (int dim : {80, 24, 100}) {
+        const int H = 4, Hkv = 2, seq_q = 19, seq_kv = 50, start = seq_kv - seq_q;
+        auto q = randn(size_t(H) * seq_q * dim, 600 + dim);                 // [H, seq_q, dim]
+        auto kh = to_half(randn(size_t(Hkv) * seq_kv * dim, 601 + dim));    // [Hkv, seq_kv, dim]
+        auto vh = to_half(randn(size_t(Hkv) * seq_kv * dim, 602 + dim));
+        OpContext ctx;
+        ctx.backend = backend();
+        ctx.inputs = {upload({H, seq_q, dim}, DataType::FP32, q), upload({Hkv, seq_kv, dim}, DataType::FP16, kh),
+                      upload({Hkv, seq_kv, dim}, DataType::FP16, vh)};
+        auto out = Tensor::allocate({H, seq_q, dim}, DataType::FP32, backend());
+        REQUIRE(out.ok());
+        ctx.outputs = {out.take()};
+        ctx.attrs.set("start_pos", int64_t(start));
+        CHECK_OK(op->execute(ctx));
+        auto got = download<float>(ctx.outputs[0]);
+        // oracle layouts: q [seq_q, H, dim], cache [Hkv, max_seq, dim] halves, out [seq_q, H * dim]
+        std::vector<float> q_tok(q.size()), want_tok(q.size()), want(q.size());
+        for (int h = 0; h < H; ++h)
+            for (int s = 0; s < seq_q; ++s)
+                std::memcpy(&q_tok[(size_t(s) * H + h) * dim], &q[(size_t(h) * seq_q + s) * dim], dim * 4);
+        go_attention_cached(q_tok.data(), kh.data(), vh.data(), want_tok.data(), nullptr, 1, seq_q, H, Hkv, dim,
+                            seq_kv, seq_kv, start, 1.0f / std::sqrt(float(dim)));
+        for (int h = 0; h < H; ++h)
+            for (int s = 0; s < seq_q; ++s)
+                std::memcpy(&want[(size_t(h) * seq_q + s) * dim], &want_tok[(size_t(s) * H + h) * dim], dim * 4);
+        CHECK(close_enough(got, want, "operator, head size without a kernel"));
+        for (auto& t : ctx.inputs) backend()->destroy_buffer(t.buffer());
+        backend()->destroy_buffer(ctx.outputs[0].buffer());
+    }
+    // beyond 128 there is nothing to pad to
+    OpContext big;
+    big.backend = backend();
+    big.inputs = {upload({2, 160}, DataType::FP32, randn(320, 1)), upload({3, 160}, DataType::FP16, to_half(randn(480, 2))),
+                  upload({3, 160}, DataType::FP16, to_half(randn(480, 3)))};
+    CHECK_CODE(op->validate(big), ErrorCode::NotImplemented);
+    for (auto& t : big.inputs) backend()->destroy_buffer(t.buffer());
 }
 
 // Causal, grouped-query, chunk at start_pos > 0 through the operator, against

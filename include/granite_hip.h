@@ -207,6 +207,16 @@ int granite_hip_paged_kv_gather(void *dst_k, void *dst_v, const void *k_cache,
                                 uint32_t num_kv_heads, uint32_t head_dim, uint32_t len,
                                 uint32_t block_size, uint32_t max_seq_len);
 
+/* Strided row copy on the launch stream: for every row r < rows, the first copy_bytes of
+ * src + r*src_row_bytes go to dst + r*dst_row_bytes and bytes copy_bytes .. fill_bytes-1 of
+ * the destination row become zero (fill_bytes >= copy_bytes; equal: a plain 2-D copy).  All
+ * byte counts, pitches and pointers are multiples of 2.  MetalAttentionOp walks mapped
+ * buffers on the host for any head size (src/operators/metal/metal_operators.mm:1262-1300);
+ * the HIP operator uses this copy to present head sizes that have no kernel zero-padded to 64
+ * or 128 and to slice the result back. */
+int granite_hip_copy_rows(void *dst, int64_t dst_row_bytes, const void *src, int64_t src_row_bytes,
+                          uint64_t rows, uint32_t copy_bytes, uint32_t fill_bytes);
+
 /* ---- attention --------------------------------------------------------- */
 
 /* MetalCompute::multihead_attention (metal_compute.h:799-816;
