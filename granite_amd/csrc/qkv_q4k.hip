@@ -28,8 +28,11 @@
 // so a nibble costs a mask, a byte shuffle and a 24-bit multiply shared between two weights,
 // and nothing is rounded; d * 2^24 is applied once per super-block to the accumulator.  The
 // minima go through one more MFMA per super-block, the integer minima against the sums of
-// the inputs of the sub-blocks.  Inputs are split into a half and a half remainder (two MFMAs
-// per step) so that float inputs lose nothing.  A workgroup stages its 512 input columns in
+// the inputs of the sub-blocks.  A token's inputs of a chunk are first divided by the power of
+// two that brings the largest of them into [1, 2) (exact; undone when the chunk's result is
+// added), then split into a half and a half remainder (two MFMAs per step): 22 significant
+// bits of the largest input and the same absolute resolution for the others, whatever the
+// magnitude of the inputs, and no sub-block sum can leave the half range.  A workgroup stages its 512 input columns in
 // LDS once (both halves, and the sub-block sums) for its 8 waves x 32 weight rows; the chunks
 // of K are combined by a second small kernel.
 #include "common.h"
@@ -222,7 +225,8 @@ constexpr int kChunkK = 512;          // input columns a workgroup stages: two s
 constexpr int kChunkBlocks = kChunkK / int(kQK);
 constexpr int kXPitch = kChunkK + 8;  // halves per token row in LDS (16-byte reads without bank conflicts)
 constexpr int kSubPerChunk = kChunkK / 32;
-constexpr size_t kTokLdsBytes = size_t(2 * kTokTile * kXPitch + 2 * kTokTile * kSubPerChunk) * sizeof(uint16_t);
+constexpr size_t kTokLdsBytes =
+    size_t(2 * kTokTile * kXPitch + 2 * kTokTile * kSubPerChunk) * sizeof(uint16_t) + kTokTile * sizeof(float);
 
 struct MatmulTokParams {
     MatvecParams m;   // x, weights and row numbering as for the matvec; m.batch = all tokens
@@ -243,6 +247,7 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
     uint16_t* const s_xl = s_xh + kTokTile * kXPitch;       // remainder of x
     uint16_t* const s_sh = s_xl + kTokTile * kXPitch;       // [kTokTile][kSubPerChunk] sub-block sums
     uint16_t* const s_sl = s_sh + kTokTile * kSubPerChunk;  // and their remainders
+    float* const s_unit = reinterpret_cast<float*>(s_sl + kTokTile * kSubPerChunk);  // [kTokTile] power of two a token's inputs were divided by
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t n = lane & 31, g = lane >> 5;
     const uint32_t chunk = blockIdx.y;
@@ -274,21 +279,41 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
             nib[sb][G] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(blk + 16 + 32 * G + 16 * g));
     }
 
-    // ---- stage the chunk's inputs: thread (token, sub-block) converts 32 floats
+    // ---- stage the chunk's inputs: thread (token, sub-block) converts 32 floats.  A token's
+    // inputs of this chunk are first scaled by a power of two (exact) that brings the largest
+    // of them into [1, 2), so that the split into a half and a half remainder keeps 22
+    // significant bits of the largest inputs whatever their magnitude -- inputs beyond the
+    // half range and inputs far below its normal range alike -- and a sub-block's sum of 32
+    // inputs stays below 64.  The factor is taken out again when the chunk's products are
+    // added to y.
     {
         const uint32_t b = tid / kSubPerChunk, j = tid % kSubPerChunk;
         const bool live = b < tile_batch && k0 + 32 * j < K;
         const float* xp = p.x + int64_t(tok0 + min(b, tile_batch - 1)) * p.x_stride + min(k0 + 32 * j, K - 32);
+        float4v raw[8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            raw[i] = *reinterpret_cast<const float4v*>(xp + 4 * i);
+            if (live) amax = fmaxf(fmaxf(amax, fmaxf(fabsf(raw[i].x), fabsf(raw[i].y))), fmaxf(fabsf(raw[i].z), fabsf(raw[i].w)));
+        }
+        static_assert(kSubPerChunk == 16, "a token's sub-blocks are 16 neighbouring lanes");
+#pragma unroll
+        for (int m = 1; m < kSubPerChunk; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
+        // 2^floor(log2 amax), kept inside [2^-126, 2^126] so that it and its inverse are normal floats
+        const uint32_t ebits = min(max(__float_as_uint(amax) & 0x7F800000u, 0x00800000u), 0x7E800000u);
+        const float unit = amax > 0.0f ? __uint_as_float(ebits) : 1.0f;
+        const float scale = 1.0f / unit;
+        if (j == 0) s_unit[b] = unit;
         float sum = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float4v a = *reinterpret_cast<const float4v*>(xp + 8 * i);
-            const float4v c = *reinterpret_cast<const float4v*>(xp + 8 * i + 4);
+            const float4v a = raw[2 * i], c = raw[2 * i + 1];
             const float v[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
             uint32_t hi[4], lo[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const float x0 = live ? v[2 * e] : 0.0f, x1 = live ? v[2 * e + 1] : 0.0f;
+                const float x0 = live ? v[2 * e] * scale : 0.0f, x1 = live ? v[2 * e + 1] * scale : 0.0f;
                 sum += x0 + x1;
                 const _Float16 h0 = static_cast<_Float16>(x0), h1 = static_cast<_Float16>(x1);
                 half2v hh, ll;
@@ -308,9 +333,12 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
     }
     __syncthreads();
 
-    float y[16];
+    float y[16], unit[16];  // register r is token 8 (r / 4) + 4 g + r % 4
 #pragma unroll
-    for (int r = 0; r < 16; r++) y[r] = 0.0f;
+    for (int r = 0; r < 16; r++) {
+        y[r] = 0.0f;
+        unit[r] = s_unit[8 * (r >> 2) + 4 * g + (r & 3)];
+    }
 #pragma unroll
     for (int sb = 0; sb < kChunkBlocks; sb++) {
         // integer scales and minima of the 8 sub-blocks (gguf.cpp:963-971)
@@ -368,7 +396,7 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
         const float d = live_block[sb] ? float(dd.x) * 16777216.0f : 0.0f;      // the integers were worth 2^-24
         const float dmin = live_block[sb] ? float(dd.y) * 16777216.0f : 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) y[r] += d * acc[r] - dmin * accm[r];
+        for (int r = 0; r < 16; r++) y[r] += (d * acc[r] - dmin * accm[r]) * unit[r];
     }
 
     // ---- this chunk's part of y: register r is token 8 (r / 4) + 4 g + r % 4, the lane's column its row

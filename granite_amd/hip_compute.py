@@ -177,6 +177,11 @@ class HipCompute:
             _p(dst_k), _p(dst_v), _p(k_cache), _p(v_cache), _p(block_table), num_kv_heads,
             head_dim, length, block_size, max_seq_len), "paged_kv_gather")
 
+    def copy_rows(self, dst, dst_row_bytes, src, src_row_bytes, rows, copy_bytes, fill_bytes) -> None:
+        """Strided row copy with the tail of every destination row zeroed (granite_hip_copy_rows)."""
+        check(self.lib.granite_hip_copy_rows(_p(dst), dst_row_bytes, _p(src), src_row_bytes, rows, copy_bytes,
+                                             fill_bytes), "copy_rows")
+
     # ---- attention (reference-shaped entry points)
     def multihead_attention(self, Q, K, V, output, num_heads, num_kv_heads, seq_q, seq_kv,
                             head_dim, scale, max_seq=0) -> None:

@@ -265,3 +265,25 @@ def test_calibration_library_runs_and_checks_arguments(gpu):
         with pytest.raises(RuntimeError):
             calibration.mfma_rate(buf, args["n_halves"], args["iterations"], shape=args["shape"],
                                   waves_per_simd=args["waves_per_simd"], mix=args["mix"])
+
+
+@pytest.mark.parametrize("rows,d,dp,esz", [(1, 4, 64, 4), (37, 80, 128, 2), (300, 24, 64, 2), (5, 100, 128, 4)])
+def test_copy_rows_pads_and_slices(gpu, rows, d, dp, esz):
+    """granite_hip_copy_rows: pad [rows, d] to [rows, dp] with zeros, slice it back; bit exact,
+    nothing written beyond the rows' fill range."""
+    say(f"copy_rows rows={rows} d={d} dp={dp} esz={esz}")
+    dt = np.uint16 if esz == 2 else np.uint32
+    rng = np.random.default_rng(rows + d)
+    src = rng.integers(1, np.iinfo(dt).max, size=(rows, d), dtype=dt)
+    padded = dev(np.full((rows, dp), 0x5A5A, dt))
+    gpu.copy_rows(padded, dp * esz, dev(src), d * esz, rows, d * esz, dp * esz)
+    gpu.sync()
+    got = padded.read(dt, (rows, dp))
+    assert np.array_equal(got[:, :d], src) and not got[:, d:].any()
+    back = dev(np.full((rows, d + 2), 0x77, dt))   # a destination with a wider pitch than the copy
+    gpu.copy_rows(back, (d + 2) * esz, padded, dp * esz, rows, d * esz, d * esz)
+    gpu.sync()
+    got = back.read(dt, (rows, d + 2))
+    assert np.array_equal(got[:, :d], src) and (got[:, d:] == 0x77).all()
+    with pytest.raises(GraniteHipError):
+        gpu.copy_rows(back, d * esz, padded, dp * esz, rows, dp * esz, d * esz)   # copy > fill

@@ -126,3 +126,57 @@ def test_batched_projection_scratch_can_be_reserved(gpu, oracle):
     gpu.sync()
     assert gpu.workspace_bytes() == held
     _check(oracle, yq.read(np.float32, (40, case.Nq)), case.x, case.wq, "yq")
+
+
+@pytest.mark.parametrize("batch", [1, 2, 3, 64, 256])
+def test_scale_fields_known_answer_on_gpu(gpu, batch):
+    """The hand-worked super-block of tests/golden/q4k_scales_kat.json through the kernels: with
+    one-hot inputs every output is one weight, and every weight of the block is a multiple of
+    0.25 below 2^11, so the results must be exact -- in the vector kernel (batch <= 2) and in
+    the matrix-core kernel (batch > 2), for all eight (scale, minimum) pairs."""
+    from test_oracle_q4k import kat_block
+    say(f"q4k scale-field known answer batch={batch}")
+    block, want = kat_block()
+    rows = 4
+    w = np.ascontiguousarray(np.tile(block[None, None], (rows, 1, 1)))        # [rows, 1, 144]
+    picks = (np.arange(batch) * 37 + 5) % 256 if batch < 256 else np.arange(256)
+    x = np.zeros((batch, 256), np.float32)
+    x[np.arange(batch), picks] = 1.0
+    y = dev(np.full((batch, rows), np.nan, np.float32))
+    gpu.matvec_q4k(dev(x), dev(w), y, 256, rows, batch=batch)
+    gpu.sync()
+    got = y.read(np.float32, (batch, rows))
+    assert np.array_equal(got, np.repeat(want[picks].astype(np.float32)[:, None], rows, axis=1))
+
+
+@pytest.mark.parametrize("magnitudes", ["large", "tiny", "mixed"])
+@pytest.mark.parametrize("batch", [3, 40])
+def test_batched_projection_input_magnitudes(gpu, oracle, magnitudes, batch):
+    """The matrix-core kernel (batch > 2) on inputs far outside the half range on either side:
+    thousands (a sub-block's sum of 32 exceeds 65504), millionths (below the smallest normal
+    half), and both in one batch and one row.  The bound has no absolute floor: it scales
+    with sum |x w|, as a float summation's does."""
+    say(f"q4k batched magnitudes={magnitudes} batch={batch}")
+    K, rows = 1024, 96
+    rng = np.random.default_rng({"large": 11, "tiny": 22, "mixed": 33}[magnitudes] + batch)
+    blocks = W.random_q4k(rng, rows, K)
+    x = rng.standard_normal((batch, K), dtype=np.float32)
+    if magnitudes == "large":
+        x = x * 3000.0 + 2500.0            # sub-block sums around 80000
+    elif magnitudes == "tiny":
+        x = x * 1e-6
+    else:
+        x[0::2] *= 1e-6                    # every other token tiny ...
+        x[1::2] *= 3000.0                  # ... the rest large,
+        x[:, K // 2:] *= 1e-3              # and the second chunk of K a thousand times smaller than the first
+    x = np.ascontiguousarray(x.astype(np.float32))
+    y = dev(np.full((batch, rows), np.nan, np.float32))
+    gpu.matvec_q4k(dev(x), dev(blocks), y, K, rows, batch=batch)
+    gpu.sync()
+    got = y.read(np.float32, (batch, rows))
+    want = oracle.matvec_q4k(x, blocks)
+    mag = _abs_dot(oracle, x, blocks)
+    bound = 8 * 2.0 ** -24 * np.sqrt(K) * mag
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.isfinite(got).all() and np.all(err <= bound), \
+        f"max err {err.max():.3e}, worst ratio to bound {np.max(err / np.maximum(bound, 1e-300)):.2f}"

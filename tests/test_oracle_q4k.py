@@ -2,11 +2,35 @@
 (src/llm/math_ops.cpp:67-103) without the GPU: the sizes the reference's own tests hold,
 ggml's packing of the 6-bit fields run backwards, hand-built blocks with closed-form
 values, an independent float64 dequantisation, and the reference's math_ops.cpp."""
+import json
+from pathlib import Path
+
 import numpy as np
 import pytest
 
 import oracle_bind
 from granite_amd import workloads as W
+
+KAT = json.loads((Path(__file__).parent / "golden" / "q4k_scales_kat.json").read_text())
+
+
+def kat_block():
+    """The fixture's super-block (144 bytes) and its 256 weights by the fixture's own rule,
+    from the hand-typed sc / m lists (not from any unpacking code)."""
+    scale_bytes = np.array([int(h, 16) for h in KAT["scale_bytes_hex"]], np.uint8)
+    qs = ((7 * np.arange(128) + 3) & 255).astype(np.uint8)
+    block = np.zeros(144, np.uint8)
+    block[0:2] = np.array([int(KAT["block"]["d_bits_hex"], 16)], np.uint16).view(np.uint8)
+    block[2:4] = np.array([int(KAT["block"]["dmin_bits_hex"], 16)], np.uint16).view(np.uint8)
+    block[4:16] = scale_bytes
+    block[16:] = qs
+    d, dmin, sc, m = KAT["block"]["d"], KAT["block"]["dmin"], KAT["sc"], KAT["m"]
+    w = np.zeros(256, np.float64)
+    for g in range(4):
+        for l in range(32):
+            w[64 * g + l] = d * sc[2 * g] * (int(qs[32 * g + l]) & 15) - dmin * m[2 * g]
+            w[64 * g + 32 + l] = d * sc[2 * g + 1] * (int(qs[32 * g + l]) >> 4) - dmin * m[2 * g + 1]
+    return block, w
 
 
 def dequant64(blocks: np.ndarray) -> np.ndarray:
@@ -106,3 +130,22 @@ def test_projection_against_float64_and_the_reference_routine(oracle):
     c = np.empty_like(cpu)
     ref.ref_matmul_transb_fp16(case.x, w16.reshape(case.Nq, case.K), c, 3, case.Nq, case.K)
     assert np.array_equal(c, cpu)   # same loop, same order: bit for bit
+
+
+def test_scale_fields_known_answer(oracle):
+    """tests/golden/q4k_scales_kat.json: twelve hand-typed scale bytes and the eight (scale,
+    minimum) pairs worked out by hand from src/model/gguf.cpp:963-971.  Pins the j >= 4
+    branch (two bits from one byte, four from another) without any packing code of this
+    repository in the loop."""
+    q = np.array([int(h, 16) for h in KAT["scale_bytes_hex"]], np.uint8)
+    sc, m = np.zeros(1, np.uint8), np.zeros(1, np.uint8)
+    for j in range(8):
+        oracle.lib.go_q4k_scale_min(j, q, sc, m)
+        assert (int(sc[0]), int(m[0])) == (KAT["sc"][j], KAT["m"][j]), j
+    # the same bytes through the vectorised restatement used elsewhere in this file
+    block, want = kat_block()
+    assert np.array_equal(dequant64(block[None]), want[None])
+    # and the whole block through the oracle's dequantisation: every value exact
+    w32, w16 = oracle.q4k_dequantize(block[None, None])
+    assert np.array_equal(w32.astype(np.float64).reshape(-1), want)
+    assert np.array_equal(w16.view(np.float16).astype(np.float64).reshape(-1), want)
