@@ -473,9 +473,9 @@ def bench_rope_append(gpu, steps, warmup, cpu):
         i = np.arange(d // 2, dtype=np.float32)
         freq = (1.0 / np.float32(10000.0) ** (2 * i / np.float32(d))).astype(np.float32)
         ang = (np.arange(positions, dtype=np.float32)[:, None] * freq[None, :]).astype(np.float32)
+        # the timed kernel's tables: built here (the angle in float as RoPECache does, src/llm/rope.cpp:5-22),
+        # not taken from the checker; both sides of the parity leg below read these same arrays
         cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
-        if oracle is not None:  # the reference's own table (libm in float)
-            cos, sin = oracle.rope_table(positions, d, 10000.0)
         nblk = (positions + bs - 1) // bs
         table = rng.permutation(nblk).astype(np.int32)
         bufs = dict(q=dev(q), k=dev(k), v=dev(v), cos=dev(cos), sin=dev(sin), t=dev(table),

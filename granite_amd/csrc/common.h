@@ -83,6 +83,20 @@ struct TimingSuppressed {
     bool was_;
 };
 
+// Kernels whose dynamic LDS exceeds the 64 KiB default need their limit raised once per
+// device (the attribute belongs to the function on one device).  `done` is the caller's
+// static flag array, one per kernel instantiation.
+constexpr int kMaxDevices = 64;
+inline int raise_dynamic_lds_limit(const void* kernel, size_t bytes, bool (&done)[kMaxDevices]) {
+    const int dev = ctx().device;
+    if (dev < 0 || dev >= kMaxDevices) return GRANITE_HIP_EINVAL;
+    if (!done[dev]) {
+        GHIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+        done[dev] = true;
+    }
+    return GRANITE_HIP_OK;
+}
+
 inline int launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? GRANITE_HIP_OK : static_cast<int>(e);

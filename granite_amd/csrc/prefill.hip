@@ -844,13 +844,8 @@ template <bool kQF32, bool kOutF32, int kRows, int kD>
 int launch_tiles(const AttnParams& p, dim3 grid) {
     auto kernel = attention_tiles_kernel<kQF32, kOutF32, kRows, kD>;
     constexpr size_t kLdsBytes = Geometry<kD>::kLdsBytes;
-    static bool configured = false;  // the tile buffers exceed the 64 KiB default limit
-    if (!configured) {
-        GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       static_cast<int>(kLdsBytes)));
-        configured = true;
-    }
+    static bool configured[kMaxDevices];  // the tile buffers exceed the 64 KiB default limit
+    if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(kernel), kLdsBytes, configured)) return rc;
     kernel<<<grid, dim3(kThreads), kLdsBytes, ctx().stream>>>(p);
     return launch_status();
 }

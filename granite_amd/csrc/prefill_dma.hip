@@ -633,12 +633,8 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
 template <bool kOutF32, bool kPaged>
 int launch_dma(const AttnParams& p, dim3 grid) {
     auto kernel = attention_tiles_dma_kernel<kOutF32, kPaged>;
-    static bool configured = false;  // the tile buffers exceed the 64 KiB default limit
-    if (!configured) {
-        GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kDmaLds)));
-        configured = true;
-    }
+    static bool configured[kMaxDevices];  // the tile buffers exceed the 64 KiB default limit
+    if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(kernel), kDmaLds, configured)) return rc;
     kernel<<<grid, dim3(kWThreads), kDmaLds, ctx().stream>>>(p);
     return launch_status();
 }

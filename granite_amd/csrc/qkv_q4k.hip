@@ -475,13 +475,10 @@ int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], v
         // from the last-level cache after the first launch when the matrices fit it)
         MatmulTokParams q{};
         q.chunks = (K + kChunkK - 1) / kChunkK;
-        static bool configured = false;  // the staged inputs exceed the 64 KiB default limit
-        if (!configured) {
-            GHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(matmul_q4k_tokens_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(kTokLdsBytes)));
-            configured = true;
-        }
+        static bool configured[kMaxDevices];  // the staged inputs exceed the 64 KiB default limit
+        if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(matmul_q4k_tokens_kernel), kTokLdsBytes,
+                                             configured))
+            return rc;
         // up to kMaxTiles tiles of kTokTile tokens per launch (grid.z), every tile streaming the
         // weights once (from the last-level cache after the first, when the matrices fit it)
         constexpr uint32_t kMaxTiles = 8;

@@ -36,7 +36,8 @@ public:
     /// blocks for all of them now (all chunks of a layer run before the next layer starts)
     /// and uploads the block table; when the pool has too few free blocks nothing is
     /// taken and AllocationFailed returned.  Contiguous: InvalidArgument on overflow
-    /// (src/llm/kv_cache.cpp:61-65).
+    /// (src/llm/kv_cache.cpp:61-65).  A prompt that is still open (begin() without finish())
+    /// is aborted first.
     [[nodiscard]] Result<void> begin(int num_tokens, uint32_t prefill_chunk_size);
 
     [[nodiscard]] int num_chunks() const { return static_cast<int>(starts_.size()); }
@@ -63,6 +64,14 @@ public:
     /// (increment on the last layer, transformer.mm:4822-4824); a paged sequence already has
     /// its length from begin().
     void finish();
+
+    /// Gives up an open prompt: a paged sequence is truncated back to base_len() (its length
+    /// was advanced by begin(), so after a failed run_chunk / run_layer it would otherwise
+    /// cover rows that were never written) and the blocks past it are freed; a contiguous
+    /// cache's length was never advanced.  A failed run_* call must be followed by abort()
+    /// (or by a new begin(), which does it).  No effect when nothing is open.
+    void abort();
+    [[nodiscard]] bool is_open() const { return open_; }
 
     /// Float -> half conversion of the appended rows: GRANITE_HIP_ROUND_NEAREST (the GPU
     /// path's, default) or GRANITE_HIP_ROUND_TRUNCATE (the CPU path's).

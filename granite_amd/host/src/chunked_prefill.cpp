@@ -65,7 +65,7 @@ Result<void> ChunkedPrefill::plan(int num_tokens, uint32_t prefill_chunk_size) {
 Result<void> ChunkedPrefill::begin(int num_tokens, uint32_t prefill_chunk_size) {
     if (!backend_) return Error(ErrorCode::InvalidState, "ChunkedPrefill not initialized");
     if (num_tokens <= 0) return Error(ErrorCode::InvalidArgument, "A prompt has at least one token");
-    open_ = false;
+    abort();  // a prompt left open (a run_* call failed and the caller starts over) gives its tokens back
     if (sequence_) {
         const int block_size = sequence_->block_manager()->block_size();
         base_ = sequence_->seq_len();
@@ -92,6 +92,11 @@ Result<void> ChunkedPrefill::begin(int num_tokens, uint32_t prefill_chunk_size) 
     GRANITE_TRY(plan(num_tokens, prefill_chunk_size));
     open_ = true;
     return {};
+}
+
+void ChunkedPrefill::abort() {
+    if (open_ && sequence_) sequence_->truncate(base_);  // frees the blocks past the old length
+    open_ = false;
 }
 
 Result<void> ChunkedPrefill::run_chunk(int layer, int chunk, Tensor& q, Tensor& k, const Tensor& v,

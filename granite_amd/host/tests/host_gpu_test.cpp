@@ -1251,6 +1251,43 @@ TEST_CASE(tree_verify_commit_then_decode_over_paged_prefix) {
     }
 }
 
+// A chunk that fails (wrong tensor shape) leaves a paged prompt open with its tokens already
+// taken; abort() gives them back, and a new begin() does the same by itself.
+TEST_CASE(chunked_prefill_abort_after_failed_chunk) {
+    REQUIRE(backend() != nullptr);
+    PagedKVConfig cfg;
+    cfg.block_size = 16;
+    cfg.num_blocks = 8;
+    cfg.num_layers = 1;
+    cfg.num_kv_heads = 2;
+    cfg.head_dim = D;
+    BlockManager mgr;
+    REQUIRE(mgr.initialize(cfg, backend()).ok());
+    PagedKVCache seq(&mgr);
+    REQUIRE(seq.append_tokens(20));  // an earlier prefix: 2 blocks
+    const int free_before = mgr.num_free_blocks();
+    ChunkedPrefill prefill;
+    REQUIRE(prefill.initialize(&seq, 8, backend()).ok());
+    REQUIRE(prefill.begin(70, 32).ok());
+    CHECK(prefill.is_open() && prefill.base_len() == 20 && seq.seq_len() == 90);
+    Tensor wrong = Tensor::allocate({5, 4, D}, DataType::FP32, backend()).take();  // the chunk has 32 rows
+    CHECK_CODE(prefill.run_chunk(0, 0, wrong, wrong, wrong, wrong, 0.1f, nullptr), ErrorCode::ShapeMismatch);
+    CHECK(prefill.is_open() && seq.seq_len() == 90);  // still covers rows nobody wrote
+    prefill.abort();
+    CHECK(!prefill.is_open() && seq.seq_len() == 20 && seq.num_blocks() == 2);
+    CHECK(mgr.num_free_blocks() == free_before);
+    prefill.abort();  // nothing open: no effect
+    CHECK(seq.seq_len() == 20);
+    // a new begin() on a prompt left open aborts it first
+    REQUIRE(prefill.begin(40, 0).ok());
+    CHECK(seq.seq_len() == 60);
+    REQUIRE(prefill.begin(10, 0).ok());
+    CHECK(prefill.base_len() == 20 && seq.seq_len() == 30);
+    prefill.finish();
+    CHECK(!prefill.is_open() && seq.seq_len() == 30);
+    backend()->destroy_buffer(wrong.buffer());
+}
+
 int main(int argc, char** argv) {
     if (!backend()) {
         std::printf("no usable gfx950 GPU: skipping\n");

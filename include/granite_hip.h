@@ -124,7 +124,7 @@ int granite_hip_event_elapsed_ms(void *start, void *stop, float *ms);
  * While enabled every launch is bracketed by two events on the launch stream.
  * Names: "kv_append", "kv_gather", "decode_stream" or "decode_splitk",
  * "decode_merge", "attention_tiles", "attention_merge", "tree_mask", "rope_append",
- * "matvec_q4k".  granite_hip_kernel_timing_names() writes the
+ * "matvec_q4k", "copy_rows".  granite_hip_kernel_timing_names() writes the
  * names seen so far, comma separated. */
 int granite_hip_enable_kernel_timing(int enable);
 int granite_hip_reset_kernel_timing(void);

@@ -189,6 +189,30 @@ void go_parallel_for(size_t n, size_t num_threads, go_work_fn fn, void *arg)
     free(tids);
 }
 
+/* Which thread of go_parallel_for ran each index, as the smallest index that thread ran
+ * (owner[i] == owner[j] iff one thread ran both): the partition as executed, for comparison
+ * with the reference's (tests only). */
+struct go_owner_probe {
+    pthread_t *ran;
+};
+static void go_owner_probe_fn(size_t i, void *arg) { ((struct go_owner_probe *)arg)->ran[i] = pthread_self(); }
+void go_parallel_for_owner(size_t n, size_t num_threads, int32_t *owner)
+{
+    struct go_owner_probe probe;
+    probe.ran = (pthread_t *)malloc((n + 1) * sizeof(pthread_t));
+    go_parallel_for(n, num_threads, go_owner_probe_fn, &probe);
+    for (size_t i = 0; i < n; i++) {
+        size_t first = i;
+        for (size_t j = 0; j < i; j++)
+            if (pthread_equal(probe.ran[j], probe.ran[i])) {
+                first = j;
+                break;
+            }
+        owner[i] = (int32_t)first;
+    }
+    free(probe.ran);
+}
+
 /* ------------------------------------------------------------------------- */
 /* KV cache append / gather                                                  */
 /* ------------------------------------------------------------------------- */

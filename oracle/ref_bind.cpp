@@ -8,6 +8,9 @@
 
 #include <atomic>
 #include <cstdint>
+#include <map>
+#include <thread>
+#include <vector>
 
 extern "C" {
 
@@ -18,13 +21,16 @@ void ref_fp16_to_fp32_array(const uint16_t* src, float* dst, size_t n) {
 }
 size_t ref_get_num_threads() { return granite::get_num_threads(); }
 
-// Runs the reference parallel_for and records which worker slot touched each
-// index (owner[i] = chunk number), so the partition can be compared.
+// Runs the reference parallel_for and records which thread ran each index, as the smallest
+// index that thread ran (owner[i] == owner[j] iff one thread ran both; the threads of a call
+// live until it joins them, so their ids are distinct).  That is the partition itself, not a
+// formula for it.
 void ref_parallel_for_owner(size_t n, size_t num_threads, int32_t* owner) {
-    size_t chunk = num_threads ? (n + num_threads - 1) / num_threads : n;
-    granite::parallel_for(n, num_threads, [owner, chunk](size_t i) {
-        owner[i] = chunk ? static_cast<int32_t>(i / chunk) : 0;
-    });
+    std::vector<std::thread::id> ran(n);
+    granite::parallel_for(n, num_threads, [&ran](size_t i) { ran[i] = std::this_thread::get_id(); });
+    std::map<std::thread::id, int32_t> first;
+    for (size_t i = 0; i < n; i++) first.emplace(ran[i], static_cast<int32_t>(i));  // keeps the smallest
+    for (size_t i = 0; i < n; i++) owner[i] = first[ran[i]];
 }
 
 // Counts calls; checks every index is visited exactly once.

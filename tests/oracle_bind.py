@@ -35,6 +35,7 @@ class Oracle:
         L.go_fp32_to_fp16_array.argtypes = [_f32p, _u16p, C.c_size_t]
         L.go_set_num_threads.argtypes = [_int]
         L.go_get_num_threads.restype = _int
+        L.go_parallel_for_owner.argtypes = [C.c_size_t, C.c_size_t, _i32p]
         L.go_kv_cache_append_f16.restype = _int
         L.go_kv_cache_append_f16.argtypes = [_u16p, _u16p, _int, _int, _int, _int, _int]
         L.go_kv_cache_append_f32.restype = _int

@@ -102,7 +102,16 @@ def test_parallel_for_partition_matches_reference(oracle):
     ref = oracle_bind.load_ref()
     if ref is None:
         pytest.skip("oracle/_ref not built (reference tree absent)")
-    for n, t in [(10, 4), (100, 8), (7, 8), (64, 64), (1000, 3), (1, 1)]:
+    for n, t in [(10, 4), (100, 8), (7, 8), (64, 64), (1000, 3), (1, 1), (9, 4), (13, 5), (1001, 16), (33, 32)]:
         visited = np.zeros(n, np.uint8)
         calls = ref.ref_parallel_for_count(n, t, visited)
         assert calls == n and np.all(visited == 1)
+        # the partition as executed: which thread ran which index, on both sides
+        ref_owner, own_owner = np.full(n, -1, np.int32), np.full(n, -1, np.int32)
+        ref.ref_parallel_for_owner(n, t, ref_owner)
+        oracle.lib.go_parallel_for_owner(n, t, own_owner)
+        assert np.array_equal(ref_owner, own_owner), (n, t)
+        # and against the closed form: serial below one item per thread, else chunks of ceil(n / t)
+        chunk = -(-n // t)
+        want = np.zeros(n, np.int32) if (t <= 1 or n < t) else (np.arange(n) // chunk * chunk).astype(np.int32)
+        assert np.array_equal(own_owner, want), (n, t)

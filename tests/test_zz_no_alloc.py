@@ -25,8 +25,21 @@ def _args(case, q_dtype, out, lse):
     return a, keep
 
 
+def _free_device_bytes(hip) -> int:
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def _timing_names(lib) -> list:
+    buf = C.create_string_buffer(4096)
+    lib.granite_hip_kernel_timing_names(buf, len(buf))
+    return sorted(n for n in buf.value.decode().split(",") if n)
+
+
 def test_static_scratch_decode_matches_the_allocating_entry_point(gpu, oracle):
     lib = _capi.load()
+    hip = C.CDLL("libamdhip64.so")
     limit = lib.granite_hip_static_scratch_bytes()
     assert limit == 32 << 20
     rng = np.random.default_rng(77)
@@ -47,9 +60,15 @@ def test_static_scratch_decode_matches_the_allocating_entry_point(gpu, oracle):
         _capi.check(lib.granite_hip_decode_workspace_required(C.byref(a_ref), C.byref(need)), "required")
         assert 0 < need.value <= limit
         _capi.check(lib.granite_hip_decode_attention(C.byref(a_ref)), "decode_attention")
-        held = lib.granite_hip_workspace_bytes()
-        _capi.check(lib.granite_hip_decode_attention_static(C.byref(a_new)), "decode_attention_static")
         gpu.sync()
+        held = lib.granite_hip_workspace_bytes()
+        # the device's free memory, to the byte, before and after: a hipMalloc or hipFree inside
+        # the call (or one pair of them that does not net out) would show
+        free_before = _free_device_bytes(hip)
+        _capi.check(lib.granite_hip_decode_attention_static(C.byref(a_new)), "decode_attention_static")
+        assert _free_device_bytes(hip) == free_before
+        gpu.sync()
+        assert _free_device_bytes(hip) == free_before
         assert lib.granite_hip_workspace_bytes() == held
         got, ref = out_new.read(np.uint32, (b, 32, 128)), out_ref.read(np.uint32, (b, 32, 128))
         assert np.array_equal(got, ref), "outputs differ from granite_hip_decode_attention"
@@ -57,6 +76,22 @@ def test_static_scratch_decode_matches_the_allocating_entry_point(gpu, oracle):
         want, _ = oracle.batched_paged_decode(case.q.astype(np.float32), case.k_pool, case.v_pool,
                                               case.block_tables, case.seq_lens, case.block_size, case.scale)
         assert_close(got.view(np.float32), want, "static-scratch decode vs oracle")
+        if call == 1:
+            # with kernel timing on, the allocating entry point records its launches (and creates
+            # events for that); the static one must record nothing
+            _capi.check(lib.granite_hip_reset_kernel_timing(), "reset timing")
+            _capi.check(lib.granite_hip_enable_kernel_timing(1), "enable timing")
+            try:
+                _capi.check(lib.granite_hip_decode_attention_static(C.byref(a_new)), "decode_attention_static")
+                gpu.sync()
+                assert _timing_names(lib) == [], "the static entry point recorded timing events"
+                _capi.check(lib.granite_hip_decode_attention(C.byref(a_ref)), "decode_attention")
+                gpu.sync()
+                assert _timing_names(lib) != []     # (the switch does work)
+            finally:
+                _capi.check(lib.granite_hip_enable_kernel_timing(0), "disable timing")
+                _capi.check(lib.granite_hip_reset_kernel_timing(), "reset timing")
+            assert np.array_equal(out_new.read(np.uint32, (b, 32, 128)), ref)
         del keep_ref, keep_new
 
 
