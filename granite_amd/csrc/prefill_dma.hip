@@ -21,10 +21,13 @@
 //   the block-table entry is a scalar load and an address is a scalar base plus a lane
 //   constant: no vector arithmetic per tile.  A ragged last tile falls back to per-lane
 //   addresses with the key index clamped.
-//     K tile: sixteen transfers of 8 keys x 128 bytes (lane i: key i & 7, 16-byte piece
-//       i >> 3 of the half row), 1152 bytes apart, so that the 16 lanes of an operand read
-//       (16 keys, one piece) fall into all 64 banks; the address of an operand is one lane
-//       register plus an immediate.
+//     K tile: sixteen transfers of 8 keys x 128 bytes, key-major (lane i: key i >> 3, so
+//       eight consecutive lanes fetch one whole 128-byte line; with the keys across the lanes
+//       instead, a transfer touched eight lines eight times over and the causal prefill ran
+//       2.4 % slower), the eight 16-byte pieces of a half row XOR-swizzled with the key's low
+//       bits and the transfers 1152 bytes apart, so that the 16 lanes of an operand read (16
+//       keys, one piece) fall into all 64 banks; the address of an operand is one of four lane
+//       registers plus an immediate.
 //     V tile: row-major 64 x 256 bytes, the four 64-byte chunks of a row XOR-swizzled with
 //       the key's low two bits, as ds_read_b64_tr_b16 wants them (see prefill.hip); a transfer
 //       is 4 keys x 256 bytes.
@@ -59,6 +62,7 @@ constexpr int kD = 128;
 #ifndef GHIP_DMA_RB
 #define GHIP_DMA_RB 1
 #endif
+
 constexpr int kRB = GHIP_DMA_RB;  // 32-row blocks per wave
 constexpr int kWaves = 8 / kRB;
 constexpr int kWBM = 256;       // query rows per workgroup
@@ -201,8 +205,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     const int64_t stride_bytes = p.a_tok_stride * 2;  // between consecutive tokens of one KV head
     const unsigned char* const k_bytes = reinterpret_cast<const unsigned char*>(p.k + size_t(kvh) * p.a_head_stride);
     const unsigned char* const v_bytes = reinterpret_cast<const unsigned char*>(p.v + size_t(kvh) * p.a_head_stride);
-    // K transfer (a, h): keys 8 a + (lane & 7) of the wave's, bytes 128 h + 16 (lane >> 3) .. + 15 of the row
-    const uint32_t k_lane_off = uint32_t((lane & 7) * stride_bytes) + 16 * (lane >> 3);
+    // K transfer (a, h): key 8 a + (lane >> 3) of the wave's, whose slot lane & 7 receives the 16-byte
+    // piece slot ^ key of half h of the row: eight consecutive lanes fetch one 128-byte line
+    const uint32_t k_lane_off = uint32_t((lane >> 3) * stride_bytes) + 16 * ((lane & 7) ^ (lane >> 3));
     // V transfer j: keys 4 j + (lane >> 4) of the wave's; the lane's slot (lane & 15) holds 16-byte
     // piece slot ^ 4 (key & 3) of the row
     const uint32_t v_swizzled = 16 * ((lane & 15) ^ (((lane >> 4) & 3) << 2));
@@ -247,8 +252,8 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         } else {
 #pragma unroll
             for (uint32_t a = 0; a < kWaveKeys / 8; a++) {
-                const uint32_t r = lane_row(tile * kWBN + kWaveKeys * wave + 8 * a + (lane & 7));
-                const unsigned char* src = k_bytes + uint64_t(r) * uint64_t(stride_bytes) + 16 * (lane >> 3);
+                const uint32_t r = lane_row(tile * kWBN + kWaveKeys * wave + 8 * a + (lane >> 3));
+                const unsigned char* src = k_bytes + uint64_t(r) * uint64_t(stride_bytes) + 16 * ((lane & 7) ^ (lane >> 3));
                 dma_lanes(dst + a * kKChunk, src);
                 dma_lanes(dst + (8 + a) * kKChunk, src + 128);
             }
@@ -271,10 +276,15 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
 
     // ---- operand addresses in LDS (bytes from s_raw).  K: key 32 sub + n is row n & 7 of the
     // transfer 4 sub + (n >> 3) (+ 8 for the second half of the row); the 16-byte piece 2 s + g
-    // of the row is piece (2 s + g) & 7 of its half.  Everything that depends on the step, the
-    // sub-tile and the buffer is an immediate.
-    const uint32_t k_lane = (n >> 3) * kKChunk + g * 128 + (n & 7) * 16;
-    const uint32_t k_lane_hi = k_lane + 2 * kKTile;  // buffers 2 and 3 (the immediate has 16 bits)
+    // of the row is piece (2 s + g) & 7 of its half and sits in slot piece ^ (n & 7): one lane
+    // register per value of s & 3.  Everything else that depends on the step, the sub-tile and
+    // the buffer is an immediate.
+    uint32_t k_lane_j[4], k_lane_hi_j[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++) {
+        k_lane_j[j] = (n >> 3) * kKChunk + (n & 7) * 128 + 16 * ((2 * j + g) ^ (n & 7));
+        k_lane_hi_j[j] = k_lane_j[j] + 2 * kKTile;
+    }
     // V^T through ds_read_b64_tr_b16, as in attention_tiles_kernel: 16-lane group q4, lane
     // 4 k4 + r4 inside it points at key 4 g + k4, head-dim elements 32 t + 16 (q4 & 1) + 8 (r4 & 1)
     // + 4 (r4 >> 1) .. + 3 (chunk t stored at t ^ (key & 3))
@@ -290,8 +300,8 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
     auto k_operand = [&](auto kb, auto sub, int s8) __attribute__((always_inline)) -> uint4v {
         constexpr int kBuf = decltype(kb)::value, kSub = decltype(sub)::value;
-        const uint32_t base = kBuf < 2 ? k_lane : k_lane_hi;
-        const uint32_t imm = (kBuf & 1) * kKTile + (s8 >> 2) * 8 * kKChunk + kSub * 4 * kKChunk + (s8 & 3) * 256;
+        const uint32_t base = kBuf < 2 ? k_lane_j[s8 & 3] : k_lane_hi_j[s8 & 3];
+        const uint32_t imm = (kBuf & 1) * kKTile + (s8 >> 2) * 8 * kKChunk + kSub * 4 * kKChunk;
         return *reinterpret_cast<const uint4v*>(s_raw + base + imm);
     };
     auto v_pair = [&](const unsigned char* vp) __attribute__((always_inline)) -> uint4v {
@@ -462,7 +472,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
 #pragma unroll
         for (int s8 = 0; s8 < kSteps; s8++) {
             const half8 a = as_half8(*reinterpret_cast<const uint4v*>(
-                s_raw + k_lane + buf * kKTile + (s8 >> 2) * 8 * kKChunk + sub * 4 * kKChunk + (s8 & 3) * 256));
+                s_raw + k_lane_j[s8 & 3] + buf * kKTile + (s8 >> 2) * 8 * kKChunk + sub * 4 * kKChunk));
 #pragma unroll
             for (int rb = 0; rb < kRB; rb++) c[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[rb][s8], c[rb], 0, 0, 0);
         }

@@ -3,14 +3,14 @@ kernel (attention_tiles_dma_kernel, the default where it applies: head size 128,
 queries, contiguous cache or blocks of a power of two >= 8 tokens) and the register-staged
 kernel it falls back to (attention_tiles_kernel, forced here with
 GRANITE_HIP_PREFILL_KERNEL=tiles).  Both against the oracle's restatement of
-src/llm/transformer.mm:1779-1840, and against each other.
+src/llm/transformer.mm:1779-1840 and :2044-2126, and against each other.
 Tolerances: outputs |d| <= 2e-3 or <= 1e-2 |ref|; lse 1e-4."""
 import os
 
 import numpy as np
 import pytest
 
-from granite_amd import F16, F32, MASK_CAUSAL, MASK_NONE
+from granite_amd import F16, F32, MASK_CAUSAL, MASK_NONE, MASK_TREE
 from granite_amd import workloads as W
 from gpu_util import assert_close, assert_lse, dev, say
 
@@ -106,3 +106,103 @@ def test_softmax_reference_moves_mid_stream(gpu, oracle, kernel):
     assert np.isfinite(got).all()
     assert_close(got, want[0], "out")
     assert_lse(got_lse, want_lse[0], "lse")
+
+
+@pytest.mark.parametrize("prefix,chunk,bs,hq,hkv,q_dtype,out_dtype,splits", [
+    (0, 1, 16, 4, 4, F16, F16, 0), (0, 33, 16, 8, 2, F32, F32, 0), (5, 64, 1, 4, 1, F16, F32, 0),
+    (127, 32, 12, 8, 2, F32, F16, 0), (128, 31, 8, 8, 8, F16, F16, 0), (129, 64, 4, 4, 2, F32, F32, 0),
+    (1000, 17, 16, 12, 3, F16, F32, 0),
+    (4096, 64, 16, 8, 2, F32, F32, 0),     # keys split over workgroups (few heads, many tiles)
+    (4100, 40, 32, 8, 1, F16, F16, 5),     # a split count that does not divide the tiles
+    (300, 64, 16, 4, 1, F16, F16, 7),      # more splits than tiles: empty shares write neutral partials
+])
+def test_short_chunk_default_kernel_and_tiles_kernel(gpu, oracle, prefix, chunk, bs, hq, hkv, q_dtype, out_dtype, splits):
+    """A chunk of at most 64 tokens (a quarter of a workgroup's rows) over a paged prefix, block
+    sizes on both sides of what the direct-to-LDS kernel takes, both query and output types,
+    split counts that do not divide the tiles and that exceed them: the kernel chosen by
+    default and the register-staged kernel against the oracle and against each other."""
+    say(f"short chunk prefix={prefix} chunk={chunk} bs={bs} hq={hq} hkv={hkv} q={q_dtype} out={out_dtype} "
+        f"splits={splits}")
+    case = W.make_chunked_prefill(seed=3 * prefix + chunk + bs, prefix_len=prefix, chunk=chunk, num_heads=hq,
+                                  num_kv_heads=hkv, block_size=bs, pool_slack=1.3)
+    total = prefix + chunk
+    dk, dv, dt = dev(case.k_pool), dev(case.v_pool), dev(case.block_table)
+    gpu.paged_kv_cache_append_ex(dev(case.k_new), dev(case.v_new), F16, hkv * 128, 128, dk, dv, dt, hkv, 128,
+                                 prefix, chunk, bs)
+    gpu.sync()
+    pool_k, pool_v = dk.read(np.uint16, case.k_pool.shape), dv.read(np.uint16, case.v_pool.shape)
+    want, want_lse = oracle.attention_paged(case.q[None].astype(np.float32), pool_k, pool_v, case.block_table, bs,
+                                            total, prefix, case.scale)
+    q_host = case.q if q_dtype == F16 else case.q.astype(np.float32)
+    odt = np.float32 if out_dtype == F32 else np.float16
+    old = os.environ.pop("GRANITE_HIP_ATTN_SPLITS", None)
+    if splits:
+        os.environ["GRANITE_HIP_ATTN_SPLITS"] = str(splits)
+    results = {}
+    try:
+        for kernel in ("default", "tiles"):
+            out, lse = dev(np.zeros((chunk, hq, 128), odt)), dev(np.zeros((hq, chunk), np.float32))
+            if kernel == "tiles":
+                os.environ["GRANITE_HIP_PREFILL_KERNEL"] = "tiles"
+            try:
+                gpu.attention(q=dev(q_host), q_dtype=q_dtype, q_tok_stride=hq * 128, q_head_stride=128, out=out,
+                              out_dtype=out_dtype, out_tok_stride=hq * 128, out_head_stride=128, lse=lse,
+                              seq_q=chunk, num_heads=hq, num_kv_heads=hkv, head_dim=128, scale=case.scale,
+                              k_cache=dk, v_cache=dv, cache_len=total, block_table=dt, block_size=bs,
+                              mask_mode=MASK_CAUSAL, start_pos=prefix)
+                gpu.sync()
+            finally:
+                os.environ.pop("GRANITE_HIP_PREFILL_KERNEL", None)
+            got, got_lse = out.read(odt, (chunk, hq, 128)).astype(np.float32), lse.read(np.float32, (hq, chunk))
+            assert_close(got, want[0], f"{kernel} out")
+            assert_lse(got_lse, want_lse[0], f"{kernel} lse")
+            results[kernel] = (got, got_lse)
+    finally:
+        os.environ.pop("GRANITE_HIP_ATTN_SPLITS", None)
+        if old is not None:
+            os.environ["GRANITE_HIP_ATTN_SPLITS"] = old
+    assert np.abs(results["default"][0] - results["tiles"][0]).max() <= 2e-3
+    assert np.abs(results["default"][1] - results["tiles"][1]).max() <= 1e-4
+
+
+@pytest.mark.parametrize("prefix,n,hq,hkv,bs,paged", [(0, 1, 4, 4, 16, True), (0, 40, 8, 2, 16, True),
+                                                     (100, 33, 8, 2, 12, True), (2000, 64, 32, 8, 16, True),
+                                                     (700, 64, 8, 2, 16, False), (4096, 20, 4, 1, 1, True)])
+def test_tree_default_kernel_and_tiles_kernel(gpu, oracle, prefix, n, hq, hkv, bs, paged):
+    """Tree attention (fp32 queries, a prefix in a paged or contiguous cache, the nodes as the
+    extra segment), launched as by default and with the register-staged kernel forced."""
+    say(f"tree kernels prefix={prefix} nodes={n} hq={hq} hkv={hkv} bs={bs} paged={paged}")
+    case = W.make_tree(seed=prefix + n, prefix_len=prefix, num_nodes=n, num_heads=hq, num_kv_heads=hkv,
+                       block_size=bs)
+    q = np.transpose(case.q, (1, 0, 2))[None]
+    kt = np.transpose(case.k_tree, (1, 0, 2))[None].astype(np.float32)
+    vt = np.transpose(case.v_tree, (1, 0, 2))[None].astype(np.float32)
+    want, want_lse = oracle.attention_tree(q, case.k_pool, case.v_pool, kt, vt, case.parents, prefix, case.scale,
+                                           table=case.block_table, block_size=bs)
+    if paged:
+        cache = dict(k_cache=dev(case.k_pool), v_cache=dev(case.v_pool), block_size=bs,
+                     block_table=dev(case.block_table) if prefix else None, max_seq=prefix)
+    else:  # the same prefix gathered into [Hkv, prefix, D]
+        rows = (case.block_table[np.arange(prefix) // bs] * bs + np.arange(prefix) % bs) if prefix else np.zeros(0, int)
+        kc = np.ascontiguousarray(np.transpose(case.k_pool[rows], (1, 0, 2)))
+        vc = np.ascontiguousarray(np.transpose(case.v_pool[rows], (1, 0, 2)))
+        cache = dict(k_cache=dev(kc), v_cache=dev(vc), max_seq=prefix)
+    results = {}
+    for kernel in ("default", "tiles"):
+        out, lse = dev(np.zeros((hq, n, 128), np.float32)), dev(np.zeros((hq, n), np.float32))
+        if kernel == "tiles":
+            os.environ["GRANITE_HIP_PREFILL_KERNEL"] = "tiles"
+        try:
+            gpu.attention(q=dev(case.q), q_dtype=F32, q_tok_stride=128, q_head_stride=n * 128, out=out, out_dtype=F32,
+                          out_tok_stride=128, out_head_stride=n * 128, lse=lse, seq_q=n, num_heads=hq,
+                          num_kv_heads=hkv, head_dim=128, scale=case.scale, cache_len=prefix,
+                          k_extra=dev(case.k_tree), v_extra=dev(case.v_tree), extra_len=n, parents=dev(case.parents),
+                          mask_mode=MASK_TREE, **cache)
+            gpu.sync()
+        finally:
+            os.environ.pop("GRANITE_HIP_PREFILL_KERNEL", None)
+        got, got_lse = out.read(np.float32, (hq, n, 128)), lse.read(np.float32, (hq, n))
+        assert_close(got, np.transpose(want[0], (1, 0, 2)), f"{kernel} out")
+        assert_lse(got_lse, want_lse[0], f"{kernel} lse")
+        results[kernel] = (got, got_lse)
+    assert np.abs(results["default"][0] - results["tiles"][0]).max() <= 2e-3
