@@ -557,6 +557,11 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         // last tile with a phase that applies (phase j_end is the last one: the second product of
         // the last sub-tile)
         uint32_t it = t_begin;
+        // Every load the compiler knows of is complete here (vmcnt(0), as the builtin so that it
+        // is visible to the compiler's own wait insertion): otherwise it carries one as pending
+        // into the loop and waits for the memory counter, i.e. for the transfers in flight, in
+        // the middle of the first phase.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         if (j_begin < j_end) {
             const uint32_t it_last = min(j_end / 2, n_tiles - 1);
             for (;;) {
