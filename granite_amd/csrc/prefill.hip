@@ -1,5 +1,10 @@
 // Causal GQA flash-attention prefill, chunked prefill over a paged cache and
-// tree-masked attention for gfx950 (MFMA, K/V tiles staged in LDS).
+// tree-masked attention for gfx950 (MFMA, K/V tiles staged in LDS): the launcher of
+// granite_hip_attention, the register-staged tiles kernel, the split-K merge and the tree
+// mask kernel.  Launches of head size 128 with half queries, no extra key segment and a
+// contiguous cache or blocks of a power of two of at least 8 tokens go to the direct-to-LDS
+// form of the tiles kernel instead (prefill_dma.hip), which shares the grid, the partial
+// layout and the merge; everything else runs the kernel of this file.
 //
 // Stands in for
 //   flash_attention_prefill     src/backend/metal/kernels/metal_shaders_attention.h:1447-1660
