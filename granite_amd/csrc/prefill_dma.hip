@@ -109,7 +109,7 @@ __device__ __forceinline__ void wait_transfers() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCount));
 }
 
-template <bool kOutF32, bool kPaged>
+template <bool kOutF32, bool kPaged, bool kHandOver>
 __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
     const uint32_t lds0 = uint32_t(uintptr_t((lds_byte*)s_raw));  // LDS address of the tile buffers
@@ -212,25 +212,35 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     // piece slot ^ 4 (key & 3) of the row
     const uint32_t v_swizzled = 16 * ((lane & 15) ^ (((lane >> 4) & 3) << 2));
     const uint32_t v_lane_off = uint32_t((lane >> 4) * stride_bytes) + v_swizzled;
-    // Block-table entries.  The keys a wave stages of a tile lie in one block, so it needs one
-    // entry per tile.  It keeps those of its next 64 tiles in an LDS region of its own (no
-    // barrier: only this wave touches it), refilled with one vector load every 64 tiles: the
-    // compiler's wait for that load also waits for the transfers in flight, which is why it is
-    // not issued per tile; a read from LDS is counted apart from them.
-    uint32_t* const s_entries = reinterpret_cast<uint32_t*>(s_raw + kEntryRegion) + wave * kEntries;
-    auto fill_entries = [&](uint32_t first_tile) __attribute__((always_inline)) {  // of tiles first_tile .. + 63
+    // Block-table entries.  The keys of a wave's share of a tile lie in one block, so a share
+    // needs one entry per tile.  Those of its next 64 tiles are kept in an LDS region of the
+    // share's own (touched only by the wave that stages the share at the time; a barrier lies
+    // between two that do), refilled with one vector load every 64 tiles: the compiler's wait for
+    // that load also waits for the transfers in flight, which is why it is not issued per tile;
+    // a read from LDS is counted apart from them.
+    // All of these take the wave `sw` whose share of a tile is meant: normally the wave itself; a
+    // wave that has run out of keys also stages the share of its partner that still computes
+    // (see the loops below).
+    uint32_t* const s_entries_all = reinterpret_cast<uint32_t*>(s_raw + kEntryRegion);
+    auto fill_entries = [&](uint32_t sw, uint32_t first_tile) __attribute__((always_inline)) {  // of tiles first_tile .. + 63
         if constexpr (kPaged) {
-            const uint32_t key = min(first_tile + lane, n_tiles - 1) * kWBN + kWaveKeys * wave;
-            s_entries[lane] = uint32_t(p.table[min(key, len_a - 1) >> p.bs_shift]);
+            const uint32_t key = min(first_tile + lane, n_tiles - 1) * kWBN + kWaveKeys * sw;
+            s_entries_all[sw * kEntries + lane] = uint32_t(p.table[min(key, len_a - 1) >> p.bs_shift]);
         }
     };
-    auto group_entry = [&](uint32_t tile) __attribute__((always_inline)) -> uint32_t {  // one value for the wave, in every lane
+    auto group_entry = [&](uint32_t sw, uint32_t tile) __attribute__((always_inline)) -> uint32_t {  // one value for the wave, in every lane
         if constexpr (!kPaged) return 0u;
-        return s_entries[(tile - t_begin) % kEntries];
+        return s_entries_all[sw * kEntries + (tile - t_begin) % kEntries];
     };
-    // row of the pool / cache that holds the wave's first key of `tile`
-    auto group_row = [&](uint32_t tile, uint32_t entry) __attribute__((always_inline)) -> uint32_t {
-        const uint32_t key = tile * kWBN + kWaveKeys * wave;
+    // the same entry straight from the table (when a wave takes a share over)
+    auto table_entry = [&](uint32_t sw, uint32_t tile) __attribute__((always_inline)) -> uint32_t {
+        if constexpr (!kPaged) return 0u;
+        const uint32_t key = min(tile, n_tiles - 1) * kWBN + kWaveKeys * sw;
+        return uint32_t(p.table[min(key, len_a - 1) >> p.bs_shift]);
+    };
+    // row of the pool / cache that holds the first key of `tile` in the share of wave sw
+    auto group_row = [&](uint32_t sw, uint32_t tile, uint32_t entry) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t key = tile * kWBN + kWaveKeys * sw;
         if constexpr (!kPaged) return key;
         return (__builtin_amdgcn_readfirstlane(entry) << p.bs_shift) + (key & (p.block_size - 1));
     };
@@ -239,9 +249,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         if constexpr (!kPaged) return key;
         return (uint32_t(p.table[key >> p.bs_shift]) << p.bs_shift) + (key & (p.block_size - 1));
     };
-    // the K (V) tile into buffer `buf`; `row` is the wave's group row (unused for a ragged tile)
-    auto stage_k = [&](uint32_t tile, uint32_t buf, uint32_t row) __attribute__((always_inline)) {
-        const uint32_t dst = lds0 + buf * kKTile + (kWaveKeys / 8) * wave * kKChunk;
+    // the share of wave sw of the K (V) tile into buffer `buf`; `row` is the share's group row
+    // (unused for a ragged tile)
+    auto stage_k = [&](uint32_t sw, uint32_t tile, uint32_t buf, uint32_t row) __attribute__((always_inline)) {
+        const uint32_t dst = lds0 + buf * kKTile + (kWaveKeys / 8) * sw * kKChunk;
         if ((tile + 1) * kWBN <= len_a) {
             const unsigned char* base = k_bytes + uint64_t(__builtin_amdgcn_readfirstlane(row)) * uint64_t(stride_bytes);
 #pragma unroll
@@ -252,15 +263,15 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         } else {
 #pragma unroll
             for (uint32_t a = 0; a < kWaveKeys / 8; a++) {
-                const uint32_t r = lane_row(tile * kWBN + kWaveKeys * wave + 8 * a + (lane >> 3));
+                const uint32_t r = lane_row(tile * kWBN + kWaveKeys * sw + 8 * a + (lane >> 3));
                 const unsigned char* src = k_bytes + uint64_t(r) * uint64_t(stride_bytes) + 16 * ((lane & 7) ^ (lane >> 3));
                 dma_lanes(dst + a * kKChunk, src);
                 dma_lanes(dst + (8 + a) * kKChunk, src + 128);
             }
         }
     };
-    auto stage_v = [&](uint32_t tile, uint32_t buf, uint32_t row) __attribute__((always_inline)) {
-        const uint32_t dst = lds0 + kVRegion + buf * kVTile + kWaveKeys * wave * 256;
+    auto stage_v = [&](uint32_t sw, uint32_t tile, uint32_t buf, uint32_t row) __attribute__((always_inline)) {
+        const uint32_t dst = lds0 + kVRegion + buf * kVTile + kWaveKeys * sw * 256;
         if ((tile + 1) * kWBN <= len_a) {
             const unsigned char* base = v_bytes + uint64_t(__builtin_amdgcn_readfirstlane(row)) * uint64_t(stride_bytes);
 #pragma unroll
@@ -268,7 +279,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         } else {
 #pragma unroll
             for (uint32_t j = 0; j < kWaveKeys / 4; j++) {
-                const uint32_t r = lane_row(tile * kWBN + kWaveKeys * wave + 4 * j + (lane >> 4));
+                const uint32_t r = lane_row(tile * kWBN + kWaveKeys * sw + 4 * j + (lane >> 4));
                 dma_lanes(dst + j * 1024, v_bytes + uint64_t(r) * uint64_t(stride_bytes) + v_swizzled);
             }
         }
@@ -480,23 +491,93 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         for (int rb = 0; rb < kRB; rb++) sacc[rb] = c[rb];
     };
 
+    // ---- who stages what.  A wave computes on tiles t_begin .. first_idle - 1 and only helps to
+    // stage afterwards.  Under the causal pairing the two runs of a workgroup end far apart, and a
+    // wave that still computes then has its SIMD to itself and is bound by its own instruction
+    // stream: from the tile on which wave w ^ kRunWaves (same SIMD, other run) has gone idle, that
+    // wave stages this wave's share of every tile as well as its own, and this wave issues no
+    // transfer at all.  Both sides derive the hand-over from the same numbers.
+    auto first_idle_of = [&](uint32_t w) __attribute__((always_inline)) -> uint32_t {
+        const bool second = w >= kRunWaves;
+        const bool live = !second || early_half < late_half;
+        const uint32_t half = causal ? (second ? early_half : late_half) : (second ? late_half : early_half);
+        const uint32_t first_row = live ? half * kHalf + kWaveRows * (w % kRunWaves) : p.seq_q;
+        uint32_t vis_end = 0;
+        if (first_row < p.seq_q) {
+            vis_end = len_a;
+            if (causal) vis_end = min(vis_end, p.start_pos + min(first_row + kWaveRows, p.seq_q));
+            vis_end = min(vis_end, n_tiles * kWBN);
+        }
+        const uint32_t end = max((vis_end + 31) / 32, j_begin);  // its j_end
+        return j_begin < end ? min(end / 2, n_tiles - 1) + 1 : t_begin;
+    };
+    // (kHandOver false: every wave stages its own share throughout, and the loop carries no test
+    // for it; the launcher says which -- handing over pays when the runs end far apart)
+    const uint32_t partner = wave ^ kRunWaves;
+    const uint32_t first_idle = first_idle_of(wave);
+    const uint32_t partner_first_idle = kHandOver ? first_idle_of(partner) : n_tiles;
+
+    // What a wave carries for a share it stages: at the start of iteration `it`, the block-table
+    // entry of tile it + 3 (whose K is staged in that iteration) and the row of tile it + 2 (whose
+    // V is).
+    struct Share {
+        uint32_t sw, entry_next, v_row;
+    };
+    // This iteration's transfers of a share: V of tile it + 2 (piece 0) and K of tile it + 3 (piece
+    // 1) into buffers vbuf, kbuf.
+    const auto stage_next = [&](Share& sh, uint32_t it, uint32_t kbuf, uint32_t vbuf, int piece) __attribute__((always_inline)) {
+        if (piece == 0 && it + 2 < n_tiles) stage_v(sh.sw, it + 2, vbuf, sh.v_row);
+        if (piece == 1 && it + 3 < n_tiles) {
+            const uint32_t row = group_row(sh.sw, it + 3, sh.entry_next);
+            stage_k(sh.sw, it + 3, kbuf, row);
+            sh.v_row = row;
+            if ((it + 4 - t_begin) % kEntries == 0) fill_entries(sh.sw, it + 4);
+            sh.entry_next = group_entry(sh.sw, it + 4);
+        }
+    };
+    // a share taken over at iteration `it`: its two values straight from the table (the LDS
+    // region of the share holds what is needed from tile it + 4 on)
+    const auto take_over = [&](uint32_t sw, uint32_t it) __attribute__((always_inline)) -> Share {
+        Share sh;
+        sh.sw = sw;
+        sh.entry_next = table_entry(sw, it + 3);
+        sh.v_row = group_row(sw, min(it + 2, n_tiles - 1), table_entry(sw, it + 2));
+        return sh;
+    };
+    // What the next iteration reads (K of it + 2, V of it + 1) was requested an iteration ago:
+    // the wave waits until no more transfers are outstanding than it issued in this iteration
+    // (`shares` shares' worth), then the barrier.
+    constexpr int kKTransfers = 2 * (kWaveKeys / 8), kVTransfers = kWaveKeys / 4;
+    static_assert(kKTransfers + kVTransfers == kTransfers);
+    const auto end_of_tile = [&](uint32_t it, uint32_t shares) __attribute__((always_inline)) {
+        const bool k_issued = it + 3 < n_tiles, v_issued = it + 2 < n_tiles;
+        if (shares == 0 || !v_issued) wait_transfers<0>();
+        else if (shares == 1 && k_issued) wait_transfers<kTransfers>();
+        else if (shares == 1) wait_transfers<kVTransfers>();
+        else if (k_issued) wait_transfers<2 * kTransfers>();
+        else wait_transfers<2 * kVTransfers>();
+        __syncthreads();
+    };
+
     if (t_begin < n_tiles) {  // uniform over the workgroup; an empty share writes a neutral partial
         // ---- prologue: K of the first three tiles and V of the first two into their buffers
-        // (tile t_begin + i lives in buffer i & 3)
-        fill_entries(t_begin);
+        // (tile t_begin + i lives in buffer i & 3); every wave its own share
+        fill_entries(wave, t_begin);
         {
             const uint32_t last = n_tiles - 1;
 #pragma unroll
             for (uint32_t i = 0; i < 3; i++) {
                 const uint32_t t = t_begin + i;
                 if (t > last) break;
-                const uint32_t row = group_row(t, group_entry(t));
-                stage_k(t, i, row);
-                if (i < 2) stage_v(t, i, row);
+                const uint32_t row = group_row(wave, t, group_entry(wave, t));
+                stage_k(wave, t, i, row);
+                if (i < 2) stage_v(wave, t, i, row);
             }
         }
-        uint32_t entry_next = group_entry(t_begin + 3);  // of the tile whose K is staged next
-        uint32_t v_row = group_row(min(t_begin + 2, n_tiles - 1), group_entry(t_begin + 2));  // V staged next
+        Share mine;
+        mine.sw = wave;
+        mine.entry_next = group_entry(wave, t_begin + 3);
+        mine.v_row = group_row(wave, min(t_begin + 2, n_tiles - 1), group_entry(wave, t_begin + 2));
         // V buffer 3 is read (against zero probabilities) before any tile has landed in it
         {
             uint4v* vclear = reinterpret_cast<uint4v*>(s_raw + kVRegion + 3 * kVTile);
@@ -518,25 +599,6 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             scores(0, 0, s0);
             if (j_begin >= j_mask) apply_mask(j_begin, s0);
         }
-        // This iteration's transfers: K of tile it + 3 and V of tile it + 2 into buffers kbuf, vbuf.
-        const auto stage_next = [&](uint32_t it, uint32_t kbuf, uint32_t vbuf, int piece) __attribute__((always_inline)) {
-
-            if (piece == 0 && it + 2 < n_tiles) stage_v(it + 2, vbuf, v_row);
-            if (piece == 1 && it + 3 < n_tiles) {
-                const uint32_t row = group_row(it + 3, entry_next);
-                stage_k(it + 3, kbuf, row);
-                v_row = row;
-                if ((it + 4 - t_begin) % kEntries == 0) fill_entries(it + 4);
-                entry_next = group_entry(it + 4);
-            }
-        };
-        // what the next iteration reads (K of it + 2, V of it + 1) was requested an iteration ago
-        const auto end_of_tile = [&](uint32_t it) __attribute__((always_inline)) {
-            if (it + 3 < n_tiles) wait_transfers<kTransfers>();
-            else if (it + 2 < n_tiles) wait_transfers<kWaveKeys / 4>();
-            else wait_transfers<0>();
-            __syncthreads();
-        };
         // ---- tiles on which this wave computes.  Tile `it` is in buffers B (K and V), K of
         // it + 1 in B + 1, V of it - 1 in B + 3.  Both phases always run (no branch around them:
         // a conditional second product costs the register allocator a second set of output
@@ -544,43 +606,56 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         auto iteration = [&](auto bc, uint32_t it) __attribute__((always_inline)) {
             constexpr int B = decltype(bc)::value;
             const uint32_t j = 2 * it;
+            const bool staging = !kHandOver || it < partner_first_idle;  // else the partner stages this wave's share
             fused_phase(IC<B>{}, IC<1>{}, IC<(B + 3) & 3>{}, IC<1>{}, j + 1 >= j_mask, j < j_end, j + 1, s1, s0,
                         p_new, p_old, [&](int slot) __attribute__((always_inline)) {
                             // (after the 10th and 12th MFMA of the first phase: measured best by 1 %)
-                            if (slot == 9) stage_next(it, (B + 3) & 3, (B + 2) & 3, 0);
-                            if (slot == 11) stage_next(it, (B + 3) & 3, (B + 2) & 3, 1);
+                            if (slot == 9 && staging) stage_next(mine, it, (B + 3) & 3, (B + 2) & 3, 0);
+                            if (slot == 11 && staging) stage_next(mine, it, (B + 3) & 3, (B + 2) & 3, 1);
                         });
             fused_phase(IC<(B + 1) & 3>{}, IC<0>{}, IC<B>{}, IC<0>{}, j + 2 >= j_mask, j + 1 < j_end, j + 2, s0, s1,
                         p_old, p_new, [](int) {});
-            end_of_tile(it);
+            end_of_tile(it, staging ? 1 : 0);
         };
-        // last tile with a phase that applies (phase j_end is the last one: the second product of
-        // the last sub-tile)
         uint32_t it = t_begin;
         // Every load the compiler knows of is complete here (vmcnt(0), as the builtin so that it
         // is visible to the compiler's own wait insertion): otherwise it carries one as pending
         // into the loop and waits for the memory counter, i.e. for the transfers in flight, in
         // the middle of the first phase.
         __builtin_amdgcn_s_waitcnt(0x0F70);
-        if (j_begin < j_end) {
-            const uint32_t it_last = min(j_end / 2, n_tiles - 1);
+        if (it < first_idle) {
             for (;;) {
                 iteration(IC<0>{}, it);
-                if (++it > it_last) break;
+                if (++it >= first_idle) break;
                 iteration(IC<1>{}, it);
-                if (++it > it_last) break;
+                if (++it >= first_idle) break;
                 iteration(IC<2>{}, it);
-                if (++it > it_last) break;
+                if (++it >= first_idle) break;
                 iteration(IC<3>{}, it);
-                if (++it > it_last) break;
+                if (++it >= first_idle) break;
             }
         }
-        // ---- tiles this wave only helps to stage (its rows see none of their keys)
-        for (; it < n_tiles; ++it) {
-            const uint32_t b = (it - t_begin) & 3;
-            stage_next(it, (b + 3) & 3, (b + 2) & 3, 0);
-            stage_next(it, (b + 3) & 3, (b + 2) & 3, 1);
-            end_of_tile(it);
+        // ---- tiles this wave only helps to stage (its rows see none of their keys): its own
+        // share, taken back if the partner had it, and the partner's while that wave computes
+        if (it < n_tiles) {
+            if constexpr (kHandOver) mine = take_over(wave, it);
+            if (kHandOver && it < partner_first_idle) {
+                Share theirs = take_over(partner, it);
+                for (; it < min(partner_first_idle, n_tiles); ++it) {
+                    const uint32_t b = (it - t_begin) & 3;
+                    stage_next(mine, it, (b + 3) & 3, (b + 2) & 3, 0);
+                    stage_next(theirs, it, (b + 3) & 3, (b + 2) & 3, 0);
+                    stage_next(mine, it, (b + 3) & 3, (b + 2) & 3, 1);
+                    stage_next(theirs, it, (b + 3) & 3, (b + 2) & 3, 1);
+                    end_of_tile(it, 2);
+                }
+            }
+            for (; it < n_tiles; ++it) {
+                const uint32_t b = (it - t_begin) & 3;
+                stage_next(mine, it, (b + 3) & 3, (b + 2) & 3, 0);
+                stage_next(mine, it, (b + 3) & 3, (b + 2) & 3, 1);
+                end_of_tile(it, 1);
+            }
         }
         // the second product of the last sub-tile, when the range ends with the last tile
         if (j_end == 2 * n_tiles && j_end > j_begin) accumulate((n_tiles - 1 - t_begin) & 3, 1, p_old);
@@ -645,13 +720,27 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
 }
 
-template <bool kOutF32, bool kPaged>
+template <bool kOutF32, bool kPaged, bool kHandOver>
 int launch_dma(const AttnParams& p, dim3 grid) {
-    auto kernel = attention_tiles_dma_kernel<kOutF32, kPaged>;
+    auto kernel = attention_tiles_dma_kernel<kOutF32, kPaged, kHandOver>;
     static bool configured[kMaxDevices];  // the tile buffers exceed the 64 KiB default limit
     if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(kernel), kDmaLds, configured)) return rc;
     kernel<<<grid, dim3(kWThreads), kDmaLds, ctx().stream>>>(p);
     return launch_status();
+}
+
+template <bool kOutF32, bool kPaged>
+int launch_dma_shape(const AttnParams& p, dim3 grid) {
+    // Under a causal mask the two runs of a workgroup end up to seq_q keys apart.  When that is
+    // a large part of the walk (a prompt from the start, a chunk longer than its prefix), the
+    // waves of the run that ends first take over the staging of the other run's shares; behind a
+    // long prefix the runs end almost together and the plain loop is the faster one (chunked
+    // prefill over 32k tokens: 0.6 % slower with the hand-over compiled in).
+    // The same holds when all the rows of a launch fit one run (at most 128 query rows): the other
+    // run's waves are idle from the start.
+    const bool hand_over =
+        (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && p.start_pos < p.seq_q) || p.seq_q <= uint32_t(kWBM / 2);
+    return hand_over ? launch_dma<kOutF32, kPaged, true>(p, grid) : launch_dma<kOutF32, kPaged, false>(p, grid);
 }
 
 }  // namespace
@@ -661,8 +750,8 @@ size_t tiles_dma_lds_bytes() { return kDmaLds; }
 int launch_tiles_dma(const AttnParams& p, dim3 grid, bool out_f32) {
     const bool paged = p.table != nullptr;
     if (paged && (p.bs_shift < 3)) return GRANITE_HIP_EUNSUPPORTED;
-    if (out_f32) return paged ? launch_dma<true, true>(p, grid) : launch_dma<true, false>(p, grid);
-    return paged ? launch_dma<false, true>(p, grid) : launch_dma<false, false>(p, grid);
+    if (out_f32) return paged ? launch_dma_shape<true, true>(p, grid) : launch_dma_shape<true, false>(p, grid);
+    return paged ? launch_dma_shape<false, true>(p, grid) : launch_dma_shape<false, false>(p, grid);
 }
 
 }  // namespace ghip

@@ -43,6 +43,11 @@ def _run(gpu, case_q, dk, dv, hq, hkv, seq_q, total, start, scale, out_dtype, ta
     (4100, 300, 16, 8, 1, F16),    # key splits (few workgroups, many tiles)
     (16000, 64, 32, 4, 1, F16),    # more than 64 tiles per wave: the block-table entries are refilled
     (20000, 40, 8, 2, 2, F32),
+    # a long prompt from position 0: the waves of a workgroup's early run go idle after a few tiles
+    # and stage the shares of the late run's waves for the rest of its walk, across two refills
+    # of the block-table entries
+    (0, 9000, 16, 2, 1, F16),
+    (300, 4500, 8, 2, 2, F32),
 ])
 def test_paged_chunk_both_kernels(gpu, oracle, prefix, chunk, bs, hq, hkv, out_dtype):
     say(f"prefill kernels paged prefix={prefix} chunk={chunk} bs={bs} hq={hq} hkv={hkv} out={out_dtype}")
