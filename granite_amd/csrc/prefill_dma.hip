@@ -38,6 +38,11 @@
 //   bookkeeping.  There is one code path: at the two ends of a wave's key range a stage that
 //   does not apply runs on whatever its buffers hold and is made harmless.
 //
+// * A wave that has run out of keys (the early run under the causal pairing, the empty run of a
+//   launch with few rows) stages its partner's share of every tile as well as its own, and the
+//   partner, alone on its SIMD and bound by its own instruction stream, issues no transfer
+//   (kHandOver; see the loops).
+//
 // Limits (the caller checks them and uses attention_tiles_kernel otherwise): head size 128,
 // half queries, no extra key segment (no tree mask), contiguous cache or paged cache with a
 // power-of-two block size >= 8.
