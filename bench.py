@@ -212,6 +212,23 @@ def bench_prefill(gpu, steps, warmup, cpu):
     }
     res["roofline"] = roofline("mfma", flops, kern["attention_tiles"][0], profiled_traffic("prefill", res["workload"]))
     res["roofline"]["kernel"] = "attention_tiles_dma_kernel"
+    # the same launch with float queries and float output, which is what the reference's callers
+    # (and ChunkedPrefill of the host layer) pass: an fp16 head and an fp16 remainder of Q, i.e.
+    # half as many MFMAs again in the scores
+    from granite_amd import F32
+    dq32, out32 = dev(c.q.astype(np.float32)), dev(np.zeros((S, hq, 128), np.float32))
+
+    def step_f32():
+        gpu.attention(q=dq32, q_dtype=F32, q_tok_stride=hq * 128, q_head_stride=128, out=out32, out_dtype=F32,
+                      out_tok_stride=hq * 128, out_head_stride=128, lse=lse, seq_q=S, num_heads=hq,
+                      num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=dk, v_cache=dv, cache_len=S,
+                      max_seq=c.max_seq, mask_mode=MASK_CAUSAL, start_pos=0)
+
+    ms32, _, kern32 = Timer(gpu).run(step_f32, warmup, steps)
+    res["float_queries"] = {"ms_per_step": round(ms32, 4), "TFLOPs": round(flops / (ms32 * 1e-3) / 1e12, 2),
+                            "kernels_ms": {k: round(v[0], 4) for k, v in kern32.items()}}
+    step()  # (the parity leg below reads the half-query result)
+    gpu.sync()
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()
@@ -263,6 +280,22 @@ def bench_chunked_prefill(gpu, steps, warmup, cpu):
     res["roofline"] = roofline("mfma", flops, kern["attention_tiles"][0],
                                profiled_traffic("chunked_prefill", res["workload"]))
     res["roofline"]["kernel"] = "attention_tiles_dma_kernel"
+    # with float queries and float output (see bench_prefill)
+    from granite_amd import F32
+    dq32, out32 = dev(c.q.astype(np.float32)), dev(np.zeros((chunk, hq, 128), np.float32))
+
+    def step_f32():
+        gpu.paged_kv_cache_append_ex(dkn, dvn, F16, hkv * 128, 128, dk, dv, dt, hkv, 128, prefix, chunk, bs)
+        gpu.attention(q=dq32, q_dtype=F32, q_tok_stride=hq * 128, q_head_stride=128, out=out32, out_dtype=F32,
+                      out_tok_stride=hq * 128, out_head_stride=128, lse=lse, seq_q=chunk, num_heads=hq,
+                      num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=dk, v_cache=dv, cache_len=total,
+                      block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
+
+    ms32, _, kern32 = Timer(gpu).run(step_f32, warmup, steps)
+    res["float_queries"] = {"ms_per_step": round(ms32, 4), "TFLOPs": round(flops / (ms32 * 1e-3) / 1e12, 2),
+                            "kernels_ms": {k: round(v[0], 4) for k, v in kern32.items()}}
+    step()
+    gpu.sync()
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()

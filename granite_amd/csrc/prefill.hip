@@ -1,7 +1,7 @@
 // Causal GQA flash-attention prefill, chunked prefill over a paged cache and
 // tree-masked attention for gfx950 (MFMA, K/V tiles staged in LDS): the launcher of
 // granite_hip_attention, the register-staged tiles kernel, the split-K merge and the tree
-// mask kernel.  Launches of head size 128 with half queries, no extra key segment and a
+// mask kernel.  Launches of head size 128 with no extra key segment and a
 // contiguous cache or blocks of a power of two of at least 8 tokens go to the direct-to-LDS
 // form of the tiles kernel instead (prefill_dma.hip), which shares the grid, the partial
 // layout and the merge; everything else runs the kernel of this file.
@@ -1002,15 +1002,15 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     const int rows = !a.block_table ? kRowsContiguous
                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
-    // The direct-to-LDS kernel (prefill_dma.hip) where it applies: head size 128, half queries,
-    // no extra key segment, contiguous rows or blocks of a power of two >= 8 tokens.
-    bool dma = D == 128 && !qf32 && a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE &&
+    // The direct-to-LDS kernel (prefill_dma.hip) where it applies: head size 128, no extra key
+    // segment, contiguous rows or blocks of a power of two >= 8 tokens.
+    bool dma = D == 128 && a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE &&
                 rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3);
     if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) dma = dma && e[0] != 't';  // "tiles": the register-staged kernel
     int rc;
     {
         KernelTimerScope timer("attention_tiles");
-        if (dma) rc = launch_tiles_dma(p, grid, of32);
+        if (dma) rc = launch_tiles_dma(p, grid, qf32, of32);
         else rc = D == 128 ? launch_tiles_types<128>(p, grid, rows, qf32, of32)
                            : launch_tiles_types<64>(p, grid, rows, qf32, of32);
     }

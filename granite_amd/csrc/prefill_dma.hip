@@ -44,8 +44,9 @@
 //   (kHandOver; see the loops).
 //
 // Limits (the caller checks them and uses attention_tiles_kernel otherwise): head size 128,
-// half queries, no extra key segment (no tree mask), contiguous cache or paged cache with a
-// power-of-two block size >= 8.
+// no extra key segment (no tree mask), contiguous cache or paged cache with a power-of-two
+// block size >= 8.  Queries fp16 or fp32 (fp32 as an fp16 head and an fp16 remainder: two MFMAs
+// per step of the scores on one K operand).
 //
 // kRB, the number of 32-row blocks a wave owns, is 1.  With 2 (-DGHIP_DMA_RB=2: four waves of
 // 64 rows, one per SIMD) an LDS operand read feeds two MFMAs; that form needs 434 registers per
@@ -114,7 +115,7 @@ __device__ __forceinline__ void wait_transfers() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCount));
 }
 
-template <bool kOutF32, bool kPaged, bool kHandOver>
+template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver>
 __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
     const uint32_t lds0 = uint32_t(uintptr_t((lds_byte*)s_raw));  // LDS address of the tile buffers
@@ -181,16 +182,38 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
 
     // ---- Q^T as B operands: lane (n, g), row block rb, step s holds Q[q0 + 32 rb + n][16 s + 8 g .. +7]
+    // (float queries: an fp16 head and an fp16 remainder, two MFMAs per step of the scores on the
+    // same K operand, so float queries lose nothing)
     half8 bq[kRB][kSteps];
+    half8 bq_lo[kQF32 ? kRB : 1][kQF32 ? kSteps : 1];
     uint32_t q_row[kRB];
 #pragma unroll
     for (int rb = 0; rb < kRB; rb++) {
         q_row[rb] = q0 + 32 * rb + n;
         const uint32_t q_ld = min(q_row[rb], p.seq_q - 1);
         const int64_t qoff = int64_t(q_ld) * p.q_tok_stride + int64_t(head) * p.q_head_stride;
-        const uint16_t* qp = static_cast<const uint16_t*>(p.q) + qoff + 8 * g;
+        if constexpr (kQF32) {
+            const float* qp = static_cast<const float*>(p.q) + qoff + 8 * g;
 #pragma unroll
-        for (int s = 0; s < kSteps; s++) bq[rb][s] = as_half8(*reinterpret_cast<const uint4v*>(qp + 16 * s));
+            for (int s = 0; s < kSteps; s++) {
+                const float4v x0 = *reinterpret_cast<const float4v*>(qp + 16 * s);
+                const float4v x1 = *reinterpret_cast<const float4v*>(qp + 16 * s + 4);
+                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                half8 hi, lo;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const _Float16 h = static_cast<_Float16>(x[i]);
+                    hi[i] = h;
+                    lo[i] = static_cast<_Float16>(x[i] - static_cast<float>(h));
+                }
+                bq[rb][s] = hi;
+                bq_lo[rb][s] = lo;
+            }
+        } else {
+            const uint16_t* qp = static_cast<const uint16_t*>(p.q) + qoff + 8 * g;
+#pragma unroll
+            for (int s = 0; s < kSteps; s++) bq[rb][s] = as_half8(*reinterpret_cast<const uint4v*>(qp + 16 * s));
+        }
     }
 
     float m_ref[kRB];  // reference maxima (log2 domain) the probabilities are relative to
@@ -442,6 +465,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
                 softmax_step(rb, s8);
                 side(kRB * s8 + rb);
                 __builtin_amdgcn_sched_barrier(0);
+                if constexpr (kQF32) {
+                    c[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ring[s8 % kRing]), bq_lo[rb][s8], c[rb], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
 #pragma unroll
@@ -490,7 +517,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             const half8 a = as_half8(*reinterpret_cast<const uint4v*>(
                 s_raw + k_lane_j[s8 & 3] + buf * kKTile + (s8 >> 2) * 8 * kKChunk + sub * 4 * kKChunk));
 #pragma unroll
-            for (int rb = 0; rb < kRB; rb++) c[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[rb][s8], c[rb], 0, 0, 0);
+            for (int rb = 0; rb < kRB; rb++) {
+                c[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq[rb][s8], c[rb], 0, 0, 0);
+                if constexpr (kQF32) c[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bq_lo[rb][s8], c[rb], 0, 0, 0);
+            }
         }
 #pragma unroll
         for (int rb = 0; rb < kRB; rb++) sacc[rb] = c[rb];
@@ -725,16 +755,16 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
 }
 
-template <bool kOutF32, bool kPaged, bool kHandOver>
+template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver>
 int launch_dma(const AttnParams& p, dim3 grid) {
-    auto kernel = attention_tiles_dma_kernel<kOutF32, kPaged, kHandOver>;
+    auto kernel = attention_tiles_dma_kernel<kQF32, kOutF32, kPaged, kHandOver>;
     static bool configured[kMaxDevices];  // the tile buffers exceed the 64 KiB default limit
     if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(kernel), kDmaLds, configured)) return rc;
     kernel<<<grid, dim3(kWThreads), kDmaLds, ctx().stream>>>(p);
     return launch_status();
 }
 
-template <bool kOutF32, bool kPaged>
+template <bool kQF32, bool kOutF32, bool kPaged>
 int launch_dma_shape(const AttnParams& p, dim3 grid) {
     // Under a causal mask the two runs of a workgroup end up to seq_q keys apart.  When that is
     // a large part of the walk (a prompt from the start, a chunk longer than its prefix), the
@@ -745,18 +775,24 @@ int launch_dma_shape(const AttnParams& p, dim3 grid) {
     // run's waves are idle from the start.
     const bool hand_over =
         (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && p.start_pos < p.seq_q) || p.seq_q <= uint32_t(kWBM / 2);
-    return hand_over ? launch_dma<kOutF32, kPaged, true>(p, grid) : launch_dma<kOutF32, kPaged, false>(p, grid);
+    return hand_over ? launch_dma<kQF32, kOutF32, kPaged, true>(p, grid)
+                     : launch_dma<kQF32, kOutF32, kPaged, false>(p, grid);
+}
+
+template <bool kQF32, bool kOutF32>
+int launch_dma_layout(const AttnParams& p, dim3 grid) {
+    return p.table != nullptr ? launch_dma_shape<kQF32, kOutF32, true>(p, grid)
+                              : launch_dma_shape<kQF32, kOutF32, false>(p, grid);
 }
 
 }  // namespace
 
 size_t tiles_dma_lds_bytes() { return kDmaLds; }
 
-int launch_tiles_dma(const AttnParams& p, dim3 grid, bool out_f32) {
-    const bool paged = p.table != nullptr;
-    if (paged && (p.bs_shift < 3)) return GRANITE_HIP_EUNSUPPORTED;
-    if (out_f32) return paged ? launch_dma_shape<true, true>(p, grid) : launch_dma_shape<true, false>(p, grid);
-    return paged ? launch_dma_shape<false, true>(p, grid) : launch_dma_shape<false, false>(p, grid);
+int launch_tiles_dma(const AttnParams& p, dim3 grid, bool q_f32, bool out_f32) {
+    if (p.table != nullptr && p.bs_shift < 3) return GRANITE_HIP_EUNSUPPORTED;
+    if (q_f32) return out_f32 ? launch_dma_layout<true, true>(p, grid) : launch_dma_layout<true, false>(p, grid);
+    return out_f32 ? launch_dma_layout<false, true>(p, grid) : launch_dma_layout<false, false>(p, grid);
 }
 
 }  // namespace ghip

@@ -44,10 +44,10 @@ struct AttnParams {
 };
 
 // The direct-to-LDS form of the tiles kernel (prefill_dma.hip): same grid, same partial-result
-// layout and same merge launch as attention_tiles_kernel.  Only for head size 128, half
-// queries, no extra key segment, and a contiguous cache or a paged one whose block size is a
-// power of two of at least 8 tokens; the caller checks that.
-int launch_tiles_dma(const AttnParams& p, dim3 grid, bool out_f32);
+// layout and same merge launch as attention_tiles_kernel.  Only for head size 128, no extra
+// key segment, and a contiguous cache or a paged one whose block size is a power of two of at
+// least 8 tokens; the caller checks that.
+int launch_tiles_dma(const AttnParams& p, dim3 grid, bool q_f32, bool out_f32);
 size_t tiles_dma_lds_bytes();
 
 }  // namespace ghip

@@ -1,6 +1,6 @@
 """GPU parity of the two prefill kernels behind granite_hip_attention: the direct-to-LDS
-kernel (attention_tiles_dma_kernel, the default where it applies: head size 128, half
-queries, contiguous cache or blocks of a power of two >= 8 tokens) and the register-staged
+kernel (attention_tiles_dma_kernel, the default where it applies: head size 128, half or
+float queries, contiguous cache or blocks of a power of two >= 8 tokens) and the register-staged
 kernel it falls back to (attention_tiles_kernel, forced here with
 GRANITE_HIP_PREFILL_KERNEL=tiles).  Both against the oracle's restatement of
 src/llm/transformer.mm:1779-1840 and :2044-2126, and against each other.
@@ -211,3 +211,48 @@ def test_tree_default_kernel_and_tiles_kernel(gpu, oracle, prefix, n, hq, hkv, b
         assert_lse(got_lse, want_lse[0], f"{kernel} lse")
         results[kernel] = (got, got_lse)
     assert np.abs(results["default"][0] - results["tiles"][0]).max() <= 2e-3
+
+
+@pytest.mark.parametrize("prefix,chunk,bs,hq,hkv,out_dtype", [
+    (0, 300, 16, 8, 2, F32),       # a prompt from position 0: the early run's waves hand over
+    (2000, 257, 32, 8, 8, F32),    # behind a prefix: the plain loop
+    (5000, 100, 8, 4, 1, F16),     # key splits; float queries with half output
+    (0, 1, 16, 4, 4, F32),
+])
+def test_float_queries_both_kernels(gpu, oracle, prefix, chunk, bs, hq, hkv, out_dtype):
+    """Float queries (what the reference's callers pass): both kernels take them as an fp16 head
+    and an fp16 remainder, so they must agree with the oracle's float arithmetic to the same
+    tolerance as half queries do -- also with queries whose remainders matter (values with 20
+    significant bits)."""
+    say(f"float queries prefix={prefix} chunk={chunk} bs={bs} hq={hq} hkv={hkv} out={out_dtype}")
+    case = W.make_chunked_prefill(seed=11 * prefix + chunk, prefix_len=prefix, chunk=chunk, num_heads=hq,
+                                  num_kv_heads=hkv, block_size=bs, pool_slack=1.3)
+    rng = np.random.default_rng(prefix + chunk)
+    q = (case.q.astype(np.float32) * (1.0 + rng.integers(-512, 512, case.q.shape).astype(np.float32) * 2.0 ** -20))
+    total = prefix + chunk
+    dk, dv, dt = dev(case.k_pool), dev(case.v_pool), dev(case.block_table)
+    gpu.paged_kv_cache_append_ex(dev(case.k_new), dev(case.v_new), F16, hkv * 128, 128, dk, dv, dt, hkv, 128,
+                                 prefix, chunk, bs)
+    gpu.sync()
+    pool_k, pool_v = dk.read(np.uint16, case.k_pool.shape), dv.read(np.uint16, case.v_pool.shape)
+    want, want_lse = oracle.attention_paged(q[None], pool_k, pool_v, case.block_table, bs, total, prefix, case.scale)
+    odt = np.float32 if out_dtype == F32 else np.float16
+    results = {}
+    for kernel in ("dma", "tiles"):
+        out, lse = dev(np.zeros((chunk, hq, 128), odt)), dev(np.zeros((hq, chunk), np.float32))
+        if kernel == "tiles":
+            os.environ["GRANITE_HIP_PREFILL_KERNEL"] = "tiles"
+        try:
+            gpu.attention(q=dev(q), q_dtype=F32, q_tok_stride=hq * 128, q_head_stride=128, out=out,
+                          out_dtype=out_dtype, out_tok_stride=hq * 128, out_head_stride=128, lse=lse, seq_q=chunk,
+                          num_heads=hq, num_kv_heads=hkv, head_dim=128, scale=case.scale, k_cache=dk, v_cache=dv,
+                          cache_len=total, block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
+            gpu.sync()
+        finally:
+            os.environ.pop("GRANITE_HIP_PREFILL_KERNEL", None)
+        got, got_lse = out.read(odt, (chunk, hq, 128)).astype(np.float32), lse.read(np.float32, (hq, chunk))
+        assert_close(got, want[0], f"{kernel} out")
+        assert_lse(got_lse, want_lse[0], f"{kernel} lse")
+        results[kernel] = (got, got_lse)
+    assert np.abs(results["dma"][0] - results["tiles"][0]).max() <= 1e-3
+    assert np.abs(results["dma"][1] - results["tiles"][1]).max() <= 1e-5
