@@ -40,6 +40,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
 CPU_SAMPLE_SECONDS = 10.0   # time box of each workload's CPU-baseline sample
+FLOAT_QUERY_LEG = True  # prefill workloads: also time the launch with float queries
 CLOCK_RAMP_MS = 100.0       # untimed work in front of every measurement, see Timer.run
 
 # HBM bytes per launch of each workload's dominant kernel, as counted by rocprofv3
@@ -224,11 +225,12 @@ def bench_prefill(gpu, steps, warmup, cpu):
                       num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=dk, v_cache=dv, cache_len=S,
                       max_seq=c.max_seq, mask_mode=MASK_CAUSAL, start_pos=0)
 
-    ms32, _, kern32 = Timer(gpu).run(step_f32, warmup, steps)
-    res["float_queries"] = {"ms_per_step": round(ms32, 4), "TFLOPs": round(flops / (ms32 * 1e-3) / 1e12, 2),
-                            "kernels_ms": {k: round(v[0], 4) for k, v in kern32.items()}}
-    step()  # (the parity leg below reads the half-query result)
-    gpu.sync()
+    if FLOAT_QUERY_LEG:
+        ms32, _, kern32 = Timer(gpu).run(step_f32, warmup, steps)
+        res["float_queries"] = {"ms_per_step": round(ms32, 4), "TFLOPs": round(flops / (ms32 * 1e-3) / 1e12, 2),
+                                "kernels_ms": {k: round(v[0], 4) for k, v in kern32.items()}}
+        step()  # (the parity leg below reads the half-query result)
+        gpu.sync()
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()
@@ -291,11 +293,12 @@ def bench_chunked_prefill(gpu, steps, warmup, cpu):
                       num_kv_heads=hkv, head_dim=128, scale=c.scale, k_cache=dk, v_cache=dv, cache_len=total,
                       block_table=dt, block_size=bs, mask_mode=MASK_CAUSAL, start_pos=prefix)
 
-    ms32, _, kern32 = Timer(gpu).run(step_f32, warmup, steps)
-    res["float_queries"] = {"ms_per_step": round(ms32, 4), "TFLOPs": round(flops / (ms32 * 1e-3) / 1e12, 2),
-                            "kernels_ms": {k: round(v[0], 4) for k, v in kern32.items()}}
-    step()
-    gpu.sync()
+    if FLOAT_QUERY_LEG:
+        ms32, _, kern32 = Timer(gpu).run(step_f32, warmup, steps)
+        res["float_queries"] = {"ms_per_step": round(ms32, 4), "TFLOPs": round(flops / (ms32 * 1e-3) / 1e12, 2),
+                                "kernels_ms": {k: round(v[0], 4) for k, v in kern32.items()}}
+        step()
+        gpu.sync()
     if cpu:
         import oracle_bind
         oracle = oracle_bind.load()
@@ -659,13 +662,16 @@ EXTRA_WORKLOADS = {"copy_calibration": bench_copy_calibration, "mfma_calibration
 
 
 def main() -> int:
-    global CLOCK_RAMP_MS
+    global CLOCK_RAMP_MS, FLOAT_QUERY_LEG
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", *WORKLOADS, *EXTRA_WORKLOADS])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--no-float-queries", action="store_true",
+                    help="prefill workloads: skip the second timing with float queries (profiling passes, so "
+                         "that every counter belongs to the half-query kernel)")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_MS,
                     help="untimed work in front of every measurement (0 for counter passes)")
     args = ap.parse_args()
@@ -675,6 +681,7 @@ def main() -> int:
         return 2
 
     CLOCK_RAMP_MS = args.ramp_ms
+    FLOAT_QUERY_LEG = not args.no_float_queries
     from granite_amd import get_hip_compute
     gpu = get_hip_compute(0)
     info = gpu.device_info()

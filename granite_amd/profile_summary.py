@@ -65,7 +65,8 @@ def trace_cmd(w: str, out: Path) -> list[str]:
         return ["rocprofv3", "--kernel-trace", "--stats", "-d", str(out / "trace"), "-o", "t", "--output-format",
                 "csv", "--", "python3", "bench.py", "--workload", w, "--steps", "2", "--no-cpu"]
     return ["rocprofv3", "--kernel-trace", "--stats", "-d", str(out / "trace"), "-o", "t", "--output-format",
-            "csv", "--", "python3", "bench.py", "--workload", w, "--steps", "20", "--warmup", "3", "--no-cpu"]
+            "csv", "--", "python3", "bench.py", "--workload", w, "--steps", "20", "--warmup", "3", "--no-cpu",
+            *(["--no-float-queries"] if w in MFMA_BOUND else [])]
 
 
 def pmc_cmd(w: str, out: Path, tag: str, counters: str) -> list[str]:
@@ -74,7 +75,7 @@ def pmc_cmd(w: str, out: Path, tag: str, counters: str) -> list[str]:
                 "--", "python3", "bench.py", "--workload", w, "--steps", "1", "--no-cpu"]
     return ["rocprofv3", "--pmc", *counters.split(), "-d", str(out / tag), "-o", "p", "--output-format", "csv",
             "--", "python3", "bench.py", "--workload", w, "--steps", "5", "--warmup", "2", "--no-cpu",
-            "--ramp-ms", "0"]
+            "--ramp-ms", "0", *(["--no-float-queries"] if w in MFMA_BOUND else [])]
 
 
 def shown(cmd: list[str]) -> str:
