@@ -623,9 +623,8 @@ def bench_qkv_q4k(gpu, steps, warmup, cpu):
                            "note": "one set of weights re-read every step: served by the last-level cache, not HBM"},
         "batch_64": {"ms_per_step": round(ms64, 4), "kernels_ms": {k: round(v[0], 4) for k, v in kern64.items()},
                      "weights_GBps": round(weights / (ms64 * 1e-3) / 1e9, 1),
-                     "note": "64 tokens on the matrix cores: two tiles of 32 tokens in one launch, each streaming "
-                             "the weights once (the second from the last-level cache, so the weights count "
-                             "once), and a launch that adds the eight chunks of K"},
+                     "note": "64 tokens on the matrix cores: one launch whose workgroups take two tiles of 32 "
+                             "tokens through each unpacked weight, and a launch that adds the eight chunks of K"},
     }
     res["roofline"] = roofline("hbm", nbytes, kern["matvec_q4k"][0], profiled_traffic("qkv_q4k", res["workload"]))
     res["roofline"]["kernel"] = "matvec_q4k_kernel"

@@ -218,21 +218,23 @@ __global__ void __launch_bounds__(kWavesPerGroup* kWave) matvec_q4k_kernel(Matve
 
 // ---- a batch of tokens on the matrix cores ---------------------------------------------------
 
-constexpr int kTokTile = 32;          // tokens per launch (rows of the A operand)
+constexpr int kTokTile = 32;          // tokens of one MFMA's A operand; a workgroup takes one or two such tiles
 constexpr int kTokWaves = 8;          // waves per workgroup, 32 weight rows each
 constexpr int kTokRows = 32 * kTokWaves;
 constexpr int kChunkK = 512;          // input columns a workgroup stages: two super-blocks
 constexpr int kChunkBlocks = kChunkK / int(kQK);
 constexpr int kXPitch = kChunkK + 8;  // halves per token row in LDS (16-byte reads without bank conflicts)
 constexpr int kSubPerChunk = kChunkK / 32;
-constexpr size_t kTokLdsBytes =
-    size_t(2 * kTokTile * kXPitch + 2 * kTokTile * kSubPerChunk) * sizeof(uint16_t) + kTokTile * sizeof(float);
+constexpr size_t tok_lds_bytes(int tiles) {
+    return size_t(tiles) *
+           (size_t(2 * kTokTile * kXPitch + 2 * kTokTile * kSubPerChunk) * sizeof(uint16_t) + kTokTile * sizeof(float));
+}
 
 struct MatmulTokParams {
     MatvecParams m;   // x, weights and row numbering as for the matvec; m.batch = all tokens
-    float* partial;   // [chunks, token tiles * kTokTile, rows_total]
+    float* partial;   // [chunks, tokens, rows_total]
     uint32_t chunks;  // ceil(K / kChunkK)
-    uint32_t tokens;  // token tiles * kTokTile
+    uint32_t tokens;  // workgroups along the tokens * tokens per workgroup
 };
 
 __device__ __forceinline__ uint32_t bytes_to_u16_pair(uint32_t bytes, bool upper) {
@@ -240,19 +242,23 @@ __device__ __forceinline__ uint32_t bytes_to_u16_pair(uint32_t bytes, bool upper
     return __builtin_amdgcn_perm(0u, bytes, upper ? 0x0c030c02u : 0x0c010c00u);
 }
 
+// kTiles tiles of kTokTile tokens per workgroup: the weights are unpacked once and meet every
+// tile's inputs, so a second tile costs its staging and its MFMAs only.
+template <int kTiles>
 __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(MatmulTokParams q) {
     const MatvecParams& p = q.m;
+    constexpr int kTokens = kTiles * kTokTile;  // tokens per workgroup
     extern __shared__ __attribute__((aligned(16))) uint16_t s_tok[];
-    uint16_t* const s_xh = s_tok;                           // [kTokTile][kXPitch] half of x
-    uint16_t* const s_xl = s_xh + kTokTile * kXPitch;       // remainder of x
-    uint16_t* const s_sh = s_xl + kTokTile * kXPitch;       // [kTokTile][kSubPerChunk] sub-block sums
-    uint16_t* const s_sl = s_sh + kTokTile * kSubPerChunk;  // and their remainders
-    float* const s_unit = reinterpret_cast<float*>(s_sl + kTokTile * kSubPerChunk);  // [kTokTile] power of two a token's inputs were divided by
+    uint16_t* const s_xh = s_tok;                          // [kTokens][kXPitch] half of x
+    uint16_t* const s_xl = s_xh + kTokens * kXPitch;       // remainder of x
+    uint16_t* const s_sh = s_xl + kTokens * kXPitch;       // [kTokens][kSubPerChunk] sub-block sums
+    uint16_t* const s_sl = s_sh + kTokens * kSubPerChunk;  // and their remainders
+    float* const s_unit = reinterpret_cast<float*>(s_sl + kTokens * kSubPerChunk);  // [kTokens] power of two a token's inputs were divided by
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t n = lane & 31, g = lane >> 5;
     const uint32_t chunk = blockIdx.y;
-    const uint32_t tok0 = blockIdx.z * kTokTile;          // first token of this workgroup's tile
-    const uint32_t tile_batch = min(p.batch - tok0, uint32_t(kTokTile));
+    const uint32_t tok0 = blockIdx.z * kTokens;           // first token of this workgroup
+    const uint32_t tile_batch = min(p.batch - tok0, uint32_t(kTokens));
     const uint32_t k0 = chunk * kChunkK;
     const uint32_t K = p.blocks_per_row * kQK;
 
@@ -264,8 +270,17 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
     const uint32_t local = rowc - (seg == 0 ? 0 : p.row_end[seg - 1]);
     const uint8_t* wrow = p.w[seg] + size_t(local) * p.blocks_per_row * kBlockBytes;
 
-    // all weight loads of the chunk are requested before anything else, so that their latency
-    // runs beside the staging of the inputs
+    // ---- all loads first, the inputs ahead of the weights: loads return in the order they were
+    // issued, so the inputs (from the last-level cache) can be converted while the weights are
+    // still on their way from HBM
+    float4v raw[kTiles][8];  // thread (token, sub-block) of each tile: 32 inputs
+#pragma unroll
+    for (int t = 0; t < kTiles; t++) {
+        const uint32_t b = t * kTokTile + tid / kSubPerChunk, j = tid % kSubPerChunk;
+        const float* xp = p.x + int64_t(tok0 + min(b, tile_batch - 1)) * p.x_stride + min(k0 + 32 * j, K - 32);
+#pragma unroll
+        for (int i = 0; i < 8; i++) raw[t][i] = *reinterpret_cast<const float4v*>(xp + 4 * i);
+    }
     uint4v head[kChunkBlocks], nib[kChunkBlocks][4];
     bool live_block[kChunkBlocks];
 #pragma unroll
@@ -286,16 +301,15 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
     // half range and inputs far below its normal range alike -- and a sub-block's sum of 32
     // inputs stays below 64.  The factor is taken out again when the chunk's products are
     // added to y.
-    {
-        const uint32_t b = tid / kSubPerChunk, j = tid % kSubPerChunk;
+#pragma unroll
+    for (int t = 0; t < kTiles; t++) {
+        const uint32_t b = t * kTokTile + tid / kSubPerChunk, j = tid % kSubPerChunk;
         const bool live = b < tile_batch && k0 + 32 * j < K;
-        const float* xp = p.x + int64_t(tok0 + min(b, tile_batch - 1)) * p.x_stride + min(k0 + 32 * j, K - 32);
-        float4v raw[8];
         float amax = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            raw[i] = *reinterpret_cast<const float4v*>(xp + 4 * i);
-            if (live) amax = fmaxf(fmaxf(amax, fmaxf(fabsf(raw[i].x), fabsf(raw[i].y))), fmaxf(fabsf(raw[i].z), fabsf(raw[i].w)));
+            const float4v v = raw[t][i];
+            if (live) amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
         }
         static_assert(kSubPerChunk == 16, "a token's sub-blocks are 16 neighbouring lanes");
 #pragma unroll
@@ -308,7 +322,7 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
         float sum = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float4v a = raw[2 * i], c = raw[2 * i + 1];
+            const float4v a = raw[t][2 * i], c = raw[t][2 * i + 1];
             const float v[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
             uint32_t hi[4], lo[4];
 #pragma unroll
@@ -333,12 +347,14 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
     }
     __syncthreads();
 
-    float y[16], unit[16];  // register r is token 8 (r / 4) + 4 g + r % 4
+    float y[kTiles][16], unit[kTiles][16];  // register r of tile t is token 32 t + 8 (r / 4) + 4 g + r % 4
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        y[r] = 0.0f;
-        unit[r] = s_unit[8 * (r >> 2) + 4 * g + (r & 3)];
-    }
+    for (int t = 0; t < kTiles; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            y[t][r] = 0.0f;
+            unit[t][r] = s_unit[t * kTokTile + 8 * (r >> 2) + 4 * g + (r & 3)];
+        }
 #pragma unroll
     for (int sb = 0; sb < kChunkBlocks; sb++) {
         // integer scales and minima of the 8 sub-blocks (gguf.cpp:963-971)
@@ -353,7 +369,9 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
                 mn[j] = (scale_byte(head[sb], j + 4) >> 4) | ((scale_byte(head[sb], j) >> 6) << 4);
             }
         }
-        float16v acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        float16v acc[kTiles];
+#pragma unroll
+        for (int t = 0; t < kTiles; t++) acc[t] = float16v{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int G = 0; G < 4; G++) {
             // the lane's 16 bytes of group G: low nibbles are inputs 64 G + 16 g + 0..15 (scale 2 G),
@@ -371,41 +389,49 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
                 bw.z = __umul24(bytes_to_u16_pair(q1, false), scale);
                 bw.w = __umul24(bytes_to_u16_pair(q1, true), scale);
                 const uint32_t kk = sb * kQK + 64 * G + (high ? 32 : 0) + 16 * g + 8 * (part & 1);
-                const half8 ah = __builtin_bit_cast(half8, *reinterpret_cast<const uint4v*>(s_xh + n * kXPitch + kk));
-                const half8 al = __builtin_bit_cast(half8, *reinterpret_cast<const uint4v*>(s_xl + n * kXPitch + kk));
                 const half8 bb = __builtin_bit_cast(half8, bw);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bb, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bb, acc, 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < kTiles; t++) {
+                    const uint32_t at = (t * kTokTile + n) * kXPitch + kk;
+                    const half8 ah = __builtin_bit_cast(half8, *reinterpret_cast<const uint4v*>(s_xh + at));
+                    const half8 al = __builtin_bit_cast(half8, *reinterpret_cast<const uint4v*>(s_xl + at));
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bb, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bb, acc[t], 0, 0, 0);
+                }
             }
         }
         // minima: sum_j min_j * (sum of the inputs of sub-block j), j on the contraction axis
-        float16v accm = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        {
-            uint4v bm = {mn[0] | (mn[1] << 16), mn[2] | (mn[3] << 16), mn[4] | (mn[5] << 16), mn[6] | (mn[7] << 16)};
-            uint4v sh = *reinterpret_cast<const uint4v*>(s_sh + n * kSubPerChunk + 8 * sb);
-            uint4v sl = *reinterpret_cast<const uint4v*>(s_sl + n * kSubPerChunk + 8 * sb);
-            if (g == 1) {  // only 8 of the 16 contraction slots are used
-                bm = uint4v{0, 0, 0, 0};
+        uint4v bm = {mn[0] | (mn[1] << 16), mn[2] | (mn[3] << 16), mn[4] | (mn[5] << 16), mn[6] | (mn[7] << 16)};
+        if (g == 1) bm = uint4v{0, 0, 0, 0};  // only 8 of the 16 contraction slots are used
+        const half2v dd = __builtin_bit_cast(half2v, head[sb].x);
+        const float d = live_block[sb] ? float(dd.x) * 16777216.0f : 0.0f;      // the integers were worth 2^-24
+        const float dmin = live_block[sb] ? float(dd.y) * 16777216.0f : 0.0f;
+#pragma unroll
+        for (int t = 0; t < kTiles; t++) {
+            float16v accm = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            uint4v sh = *reinterpret_cast<const uint4v*>(s_sh + (t * kTokTile + n) * kSubPerChunk + 8 * sb);
+            uint4v sl = *reinterpret_cast<const uint4v*>(s_sl + (t * kTokTile + n) * kSubPerChunk + 8 * sb);
+            if (g == 1) {
                 sh = uint4v{0, 0, 0, 0};
                 sl = uint4v{0, 0, 0, 0};
             }
             accm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, sh), __builtin_bit_cast(half8, bm), accm, 0, 0, 0);
             accm = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, sl), __builtin_bit_cast(half8, bm), accm, 0, 0, 0);
-        }
-        const half2v dd = __builtin_bit_cast(half2v, head[sb].x);
-        const float d = live_block[sb] ? float(dd.x) * 16777216.0f : 0.0f;      // the integers were worth 2^-24
-        const float dmin = live_block[sb] ? float(dd.y) * 16777216.0f : 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) y[r] += (d * acc[r] - dmin * accm[r]) * unit[r];
+            for (int r = 0; r < 16; r++) y[t][r] += (d * acc[t][r] - dmin * accm[r]) * unit[t][r];
+        }
     }
 
-    // ---- this chunk's part of y: register r is token 8 (r / 4) + 4 g + r % 4, the lane's column its row
+    // ---- this chunk's part of y: register r of tile t is token 32 t + 8 (r / 4) + 4 g + r % 4, the
+    // lane's column its row
     if (row < rows_total) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const uint32_t b = 8 * (r >> 2) + 4 * g + (r & 3);
-            if (b < tile_batch) q.partial[(size_t(chunk) * q.tokens + tok0 + b) * rows_total + row] = y[r];
-        }
+        for (int t = 0; t < kTiles; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t b = t * kTokTile + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (b < tile_batch) q.partial[(size_t(chunk) * q.tokens + tok0 + b) * rows_total + row] = y[t][r];
+            }
     }
 }
 
@@ -430,6 +456,14 @@ __global__ void __launch_bounds__(256) matmul_q4k_tokens_merge_kernel(MatmulTokP
     p.y[seg][int64_t(b) * p.y_stride[seg] + local] = sum;
 }
 
+// Tokens per launch of the matrix-core kernel, and the token count a launch's chunk sums are
+// laid out for: whole workgroups of one tile (up to kTokTile tokens) or of two.
+constexpr uint32_t kMaxLaunchTokens = 8 * kTokTile;
+inline uint32_t padded_tokens(uint32_t batch) {
+    const uint32_t per_group = batch > uint32_t(kTokTile) ? 2 * kTokTile : kTokTile;
+    return (batch + per_group - 1) / per_group * per_group;
+}
+
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
 }  // namespace
@@ -438,9 +472,7 @@ inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 // of the matrix-core path; none for the vector kernel).
 size_t matvec_q4k_scratch_bytes(uint32_t K, uint64_t rows, uint32_t batch) {
     if (batch <= uint32_t(kMaxBatch) || K == 0) return 0;
-    constexpr uint32_t kMaxTiles = 8;
-    const uint32_t tiles = min((batch + kTokTile - 1) / kTokTile, kMaxTiles);
-    return size_t((K + kChunkK - 1) / kChunkK) * tiles * kTokTile * rows * sizeof(float);
+    return size_t((K + kChunkK - 1) / kChunkK) * padded_tokens(min(batch, kMaxLaunchTokens)) * rows * sizeof(float);
 }
 
 int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], void* const y[3],
@@ -471,21 +503,23 @@ int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], v
     const dim3 grid(uint32_t((rows + rows_per_group - 1) / rows_per_group)), block(kWavesPerGroup * kWave);
     hipStream_t st = ctx().stream;
     if (batch > uint32_t(kMaxBatch)) {
-        // a batch of tokens: the matrix cores, kTokTile tokens per launch (the weights come
-        // from the last-level cache after the first launch when the matrices fit it)
+        // a batch of tokens: the matrix cores.  Up to kMaxLaunchTokens tokens per launch, in
+        // workgroups of two tiles of kTokTile tokens (of one tile when there are no more than
+        // kTokTile); the workgroups along the tokens (grid.z) each stream the weights once, from
+        // the last-level cache after the first when the matrices fit it.
         MatmulTokParams q{};
         q.chunks = (K + kChunkK - 1) / kChunkK;
-        static bool configured[kMaxDevices];  // the staged inputs exceed the 64 KiB default limit
-        if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(matmul_q4k_tokens_kernel), kTokLdsBytes,
-                                             configured))
+        static bool configured1[kMaxDevices], configured2[kMaxDevices];  // the staged inputs exceed the 64 KiB default limit
+        if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(matmul_q4k_tokens_kernel<1>), tok_lds_bytes(1),
+                                             configured1))
             return rc;
-        // up to kMaxTiles tiles of kTokTile tokens per launch (grid.z), every tile streaming the
-        // weights once (from the last-level cache after the first, when the matrices fit it)
-        constexpr uint32_t kMaxTiles = 8;
-        for (uint32_t b0 = 0; b0 < batch; b0 += kMaxTiles * kTokTile) {
-            const uint32_t nb = min(batch - b0, kMaxTiles * uint32_t(kTokTile));
-            const uint32_t tiles = (nb + kTokTile - 1) / kTokTile;
-            q.tokens = tiles * kTokTile;
+        if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(matmul_q4k_tokens_kernel<2>), tok_lds_bytes(2),
+                                             configured2))
+            return rc;
+        for (uint32_t b0 = 0; b0 < batch; b0 += kMaxLaunchTokens) {
+            const uint32_t nb = min(batch - b0, kMaxLaunchTokens);
+            const uint32_t per_group = nb > uint32_t(kTokTile) ? 2 * kTokTile : kTokTile;
+            q.tokens = padded_tokens(nb);
             int rc = ensure_workspace(matvec_q4k_scratch_bytes(K, rows, nb));
             if (rc != GRANITE_HIP_OK) return rc;
             q.partial = static_cast<float*>(ctx().workspace);
@@ -497,8 +531,11 @@ int launch_matvec_q4k(const void* x, int64_t x_stride, const void* const w[3], v
             q.m.batch = nb;
             {
                 KernelTimerScope timer("matmul_q4k_tokens");
-                matmul_q4k_tokens_kernel<<<dim3(uint32_t((rows + kTokRows - 1) / kTokRows), q.chunks, tiles),
-                                           dim3(kTokWaves * kWave), kTokLdsBytes, st>>>(q);
+                const dim3 tgrid(uint32_t((rows + kTokRows - 1) / kTokRows), q.chunks, q.tokens / per_group);
+                if (per_group == uint32_t(kTokTile))
+                    matmul_q4k_tokens_kernel<1><<<tgrid, dim3(kTokWaves * kWave), tok_lds_bytes(1), st>>>(q);
+                else
+                    matmul_q4k_tokens_kernel<2><<<tgrid, dim3(kTokWaves * kWave), tok_lds_bytes(2), st>>>(q);
             }
             rc = launch_status();
             if (rc != GRANITE_HIP_OK) return rc;

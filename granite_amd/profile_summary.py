@@ -143,11 +143,18 @@ def main_shape_duration(w: str):
 
 
 def resources(w: str) -> dict:
+    """Registers, LDS and scratch per kernel: from the kernel trace, or from the FETCH_SIZE pass
+    (the same columns) when the trace of a workload with many launches was too large to keep."""
     res = {}
     for f in glob.glob(str(RAW / w / "trace" / "**" / "*kernel_trace.csv"), recursive=True):
         for r in csv.DictReader(open(f)):
             res[short(r["Kernel_Name"])] = (r["VGPR_Count"], r["Accum_VGPR_Count"], r["SGPR_Count"],
                                             r["LDS_Block_Size"], r["Scratch_Size"], r["Workgroup_Size_X"])
+    if not res:
+        for f in glob.glob(str(RAW / w / "fetch" / "**" / "*counter_collection.csv"), recursive=True):
+            for r in csv.DictReader(open(f)):
+                res[short(r["Kernel_Name"])] = (r["VGPR_Count"], r["Accum_VGPR_Count"], r["SGPR_Count"],
+                                                r["LDS_Block_Size"], r["Scratch_Size"], r["Workgroup_Size"])
     return res
 
 

@@ -45,7 +45,10 @@ def _check(oracle, got, x, blocks, what):
                                                             (1024, 4, 4, 32, 4), (768, 2, 1, 40, 7),
                                                             # batches of tokens: the matrix-core kernel
                                                             (256, 1, 1, 8, 5), (4096, 32, 8, 128, 64),
-                                                            (1280, 3, 1, 88, 33), (2048, 8, 2, 128, 32), (512, 2, 2, 16, 300)])
+                                                            (1280, 3, 1, 88, 33), (2048, 8, 2, 128, 32), (512, 2, 2, 16, 300),
+                                                            # workgroups of two token tiles: ragged second tile, ragged
+                                                            # last workgroup, K not a multiple of the staged chunk
+                                                            (768, 2, 1, 40, 65), (1280, 3, 1, 88, 97), (2304, 4, 2, 64, 129)])
 def test_fused_qkv_matvec_q4k(gpu, oracle, K, heads, kv_heads, head_dim, batch):
     say(f"fused qkv q4k K={K} heads={heads} kv_heads={kv_heads} head_dim={head_dim} batch={batch}")
     case = W.make_qkv_projection(seed=K + heads + batch, K=K, num_heads=heads, num_kv_heads=kv_heads,
