@@ -14,15 +14,17 @@
 // 64 lanes cover 8 super-blocks at a time, 8 lanes per block; a lane takes one 16-byte piece
 // of a block's nibbles (16 weights from the low nibbles and, 32 positions further on, 16
 // from the high ones) and the block's 16-byte header, so every load instruction of the wave
-// covers 8 x 144 contiguous bytes of a row.  The 32 inputs a lane needs are loaded once and
-// serve all its rows.  As in the reference kernel the minima are applied to the sum of the
+// covers 8 x 144 contiguous bytes of a row.  The inputs reach the lanes through LDS: the
+// workgroup loads the columns of a trip once (issued ahead of the weights' loads, so that
+// they are staged while the weights are on their way) and a lane reads the 32 it needs,
+// which serve all its rows.  As in the reference kernel the minima are applied to the sum of the
 // inputs of a sub-block instead of to every weight, and a nibble is converted with one
 // byte-to-float instruction (the high nibbles stay multiplied by 16, which the scale takes
 // back).  Lanes are combined with shuffles at the end; results are float.
 //
 // A batch of tokens (a batched decode step) goes through the matrix cores instead
-// (matmul_q4k_tokens_kernel): up to 32 tokens per launch are the rows of the MFMA's A operand,
-// 32 weight rows its columns.  What makes that cheap for a 4-bit format: the B operand is not a
+// (matmul_q4k_tokens_kernel): 32 tokens are the rows of the MFMA's A operand, 32 weight rows
+// its columns; a workgroup takes one such tile of tokens, or two through every unpacked weight.  What makes that cheap for a 4-bit format: the B operand is not a
 // dequantised weight but the integer scale * q (at most 63 * 15 = 945), written as the raw
 // bits of a half -- a denormal, i.e. exactly scale * q * 2^-24, which the matrix cores keep --
 // so a nibble costs a mask, a byte shuffle and a 24-bit multiply shared between two weights,
@@ -60,8 +62,17 @@ struct MatvecParams {
 };
 
 __device__ __forceinline__ float ubyte_to_float(uint32_t word, int byte) {
-    // compiles to v_cvt_f32_ubyte{0..3}: one instruction per byte
+    // one v_cvt_f32_ubyte{0..3} per byte
     return float((word >> (8 * byte)) & 0xFFu);
+}
+
+// `word` as the compiler must take it: a value it knows nothing about.  The nibble masks go
+// through this before their bytes are converted, because from a byte of (w & 0x0F0F0F0F) the
+// compiler otherwise makes a four-bit field extract followed by a conversion, two
+// instructions where v_cvt_f32_ubyteN on the masked word is one.  No instruction is emitted.
+__device__ __forceinline__ uint32_t opaque(uint32_t word) {
+    asm("" : "+v"(word));
+    return word;
 }
 
 // Byte k (0..11) of the 12 scale bytes held in three words.
@@ -92,7 +103,7 @@ __global__ void __launch_bounds__(kWavesPerGroup* kWave) matvec_q4k_kernel(Matve
     const uint32_t blk_lane = lane >> 3;  // block inside the group of 8 the wave covers
     const uint32_t row0 = (blockIdx.x * kWavesPerGroup + wave) * kRowsPerWave;
     const uint32_t rows_total = p.row_end[2];
-    if (row0 >= rows_total) return;
+    // (a wave past the last row stays for the barriers: its loads are clamped, its stores masked)
 
     // where each of the wave's rows lives
     const uint8_t* wrow[kRowsPerWave];
@@ -121,36 +132,74 @@ __global__ void __launch_bounds__(kWavesPerGroup* kWave) matvec_q4k_kernel(Matve
         for (int b = 0; b < kBatch; b++) acc[r][b] = 0.0f;
 
     // kGroups groups of 8 super-blocks per trip, all their loads issued before any arithmetic
-    // (one input vector: two groups, which is the whole row of a 4096-wide layer)
+    // (one input vector: two groups, which is the whole row of a 4096-wide layer).  The inputs
+    // of a trip's columns reach the lanes through LDS: the workgroup loads the slice once, 16
+    // bytes per thread and load, instead of every wave loading all of it (which was three
+    // times the bytes of the weights through the vector cache).  Their loads are issued ahead
+    // of the weights' -- loads return in issue order, so the slice (from the last-level cache)
+    // is in LDS while the weights are still on their way.  Two buffers, so that one barrier
+    // per trip is enough.
     constexpr int kGroups = kBatch == 1 ? 2 : 1;
-    for (uint32_t ib0 = 0; ib0 < p.blocks_per_row; ib0 += 8 * kGroups) {
+    constexpr uint32_t kSlice = 8 * kGroups * kQK;                    // columns per trip
+    constexpr uint32_t kSlicePad = kSlice + kSlice / 16 + kSlice / 16;  // floats per staged slice
+    constexpr int kSliceLoads = int(kSlice / 4 / (kWavesPerGroup * kWave));  // float4 per thread and input vector
+    static_assert(kSlice % (4 * kWavesPerGroup * kWave) == 0, "a slice is whole rounds of the workgroup's 16-byte loads");
+    // float idx of a slice sits at idx + 4 (idx / 64) + 16 (idx / 256): the 16 lanes that a
+    // 16-byte LDS read serves at a time (two blocks x eight pieces) then fall on 16 different
+    // groups of four banks
+    auto staged = [](uint32_t idx) { return idx + 4 * (idx / 64) + 16 * (idx / 256); };
+    __shared__ __attribute__((aligned(16))) float s_x[2][kBatch * kSlicePad];
+    const uint32_t K = p.blocks_per_row * kQK;
+    uint32_t buf = 0;
+    for (uint32_t ib0 = 0; ib0 < p.blocks_per_row; ib0 += 8 * kGroups, buf ^= 1) {
         bool live[kGroups];
         uint4v head[kGroups][kRowsPerWave], nib[kGroups][kRowsPerWave];
         float4v xlo[kGroups][kBatch][4], xhi[kGroups][kBatch][4];
+        // the trip's slice of the inputs (columns past K repeat the last four: their blocks are not live)
+        float4v slice[kBatch][kSliceLoads];
+#pragma unroll
+        for (int b = 0; b < kBatch; b++) {
+            // (an input vector past the batch repeats the last one; its results are not stored)
+            const float* xb = p.x + int64_t(min(uint32_t(b), p.batch - 1)) * p.x_stride;
+#pragma unroll
+            for (int j = 0; j < kSliceLoads; j++) {
+                const uint32_t idx = 4 * (threadIdx.x + kWavesPerGroup * kWave * j);
+                slice[b][j] = *reinterpret_cast<const float4v*>(xb + min(ib0 * kQK + idx, K - 4));
+            }
+        }
+        // the weights of all rows: these are the loads that go to memory
 #pragma unroll
         for (int gi = 0; gi < kGroups; gi++) {
             const uint32_t ib = ib0 + 8 * gi + blk_lane;
             live[gi] = ib < p.blocks_per_row;
             const uint32_t ibc = live[gi] ? ib : p.blocks_per_row - 1;
-            // weights of all rows first: these are the loads that go to memory
 #pragma unroll
             for (int r = 0; r < kRowsPerWave; r++) {
                 const uint8_t* blk = wrow[r] + size_t(ibc) * kBlockBytes;
                 head[gi][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(blk));
                 nib[gi][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(blk + 16 + 16 * piece));
             }
-            // the inputs: 16 + 16 floats per input vector
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; b++)
+#pragma unroll
+            for (int j = 0; j < kSliceLoads; j++) {
+                const uint32_t idx = 4 * (threadIdx.x + kWavesPerGroup * kWave * j);
+                *reinterpret_cast<float4v*>(&s_x[buf][b * kSlicePad + staged(idx)]) = slice[b][j];
+            }
+        __syncthreads();
+        // the lane's inputs: 16 + 16 floats per input vector and group
+#pragma unroll
+        for (int gi = 0; gi < kGroups; gi++)
 #pragma unroll
             for (int b = 0; b < kBatch; b++) {
-                // (an input vector past the batch repeats the last one; its results are not stored)
-                const float* xp = p.x + int64_t(min(uint32_t(b), p.batch - 1)) * p.x_stride + size_t(ibc) * kQK + col;
+                const float* xp = &s_x[buf][b * kSlicePad + staged((8 * gi + blk_lane) * kQK + col)];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     xlo[gi][b][i] = *reinterpret_cast<const float4v*>(xp + 4 * i);
                     xhi[gi][b][i] = *reinterpret_cast<const float4v*>(xp + 32 + 4 * i);
                 }
             }
-        }
 #pragma unroll
         for (int gi = 0; gi < kGroups; gi++) {
             // sums of the inputs of the two sub-blocks, for the minima
@@ -180,8 +229,8 @@ __global__ void __launch_bounds__(kWavesPerGroup* kWave) matvec_q4k_kernel(Matve
                 for (int b = 0; b < kBatch; b++) dot_l[b] = dot_h[b] = 0.0f;
 #pragma unroll
                 for (int wd = 0; wd < 4; wd++) {
-                    const uint32_t lo = nib[gi][r][wd] & 0x0F0F0F0Fu;
-                    const uint32_t hi = nib[gi][r][wd] & 0xF0F0F0F0u;  // 16 x the high nibbles
+                    const uint32_t lo = opaque(nib[gi][r][wd] & 0x0F0F0F0Fu);
+                    const uint32_t hi = opaque(nib[gi][r][wd] & 0xF0F0F0F0u);  // 16 x the high nibbles
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const float ql = ubyte_to_float(lo, e);
