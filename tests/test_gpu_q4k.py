@@ -48,7 +48,12 @@ def _check(oracle, got, x, blocks, what):
                                                             (1280, 3, 1, 88, 33), (2048, 8, 2, 128, 32), (512, 2, 2, 16, 300),
                                                             # workgroups of two token tiles: ragged second tile, ragged
                                                             # last workgroup, K not a multiple of the staged chunk
-                                                            (768, 2, 1, 40, 65), (1280, 3, 1, 88, 97), (2304, 4, 2, 64, 129)])
+                                                            (768, 2, 1, 40, 65), (1280, 3, 1, 88, 97), (2304, 4, 2, 64, 129),
+                                                            # rows longer than one staged slice of the inputs (4096
+                                                            # columns with one vector, 2048 with two): several trips,
+                                                            # the last one ragged
+                                                            (8448, 2, 1, 32, 1), (4352, 2, 1, 32, 2), (14336, 1, 1, 64, 1),
+                                                            (6144, 3, 3, 16, 2)])
 def test_fused_qkv_matvec_q4k(gpu, oracle, K, heads, kv_heads, head_dim, batch):
     say(f"fused qkv q4k K={K} heads={heads} kv_heads={kv_heads} head_dim={head_dim} batch={batch}")
     case = W.make_qkv_projection(seed=K + heads + batch, K=K, num_heads=heads, num_kv_heads=kv_heads,
