@@ -430,12 +430,15 @@ int granite_hip_fused_qkv_matvec_q4k(const void *x, const void *wq, const void *
  * x_stride floats apart, yq [batch, Nq] rows yq_stride apart, yk and yv
  * [batch, Nkv] rows ykv_stride apart -- the layouts granite_hip_rope_append
  * takes as q, k and v.  Up to two tokens go through the vector kernel of the
- * single-token form; more go through the matrix cores, 32 tokens per pass over
- * the weights, the inputs split into a half and a half remainder (so |x| must
- * stay below the largest half, 65504) and the 4-bit values multiplied as exact
- * integers: results are float sums of exact products, as in the other form.
- * The chunks of K are added by a second launch through the library's scratch
- * (chunks x batch x (Nq + 2 Nkv) floats). */
+ * single-token form; more go through the matrix cores, up to 64 tokens per pass
+ * over the weights, a token's inputs of a 512-column chunk scaled by a power of
+ * two into the middle of the half range and split into a half and a half
+ * remainder (inputs of any float magnitude keep 22 bits of the chunk's largest)
+ * and the 4-bit values multiplied as exact integers: results are float sums of
+ * exact products, as in the other form.  The chunks of K are added by a second
+ * launch through the library's scratch (chunks x batch, rounded up to whole
+ * workgroups of 32 or 64 tokens, x (Nq + 2 Nkv) floats:
+ * granite_hip_q4k_workspace_required). */
 int granite_hip_fused_qkv_matvec_q4k_batched(const void *x, int64_t x_stride, const void *wq,
                                              const void *wk, const void *wv, void *yq, void *yk,
                                              void *yv, int64_t yq_stride, int64_t ykv_stride,
