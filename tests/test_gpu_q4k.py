@@ -69,6 +69,30 @@ def test_fused_qkv_matvec_q4k(gpu, oracle, K, heads, kv_heads, head_dim, batch):
     _check(oracle, yv.read(np.float32, (batch, case.Nkv)), case.x, case.wv, "yv")
 
 
+@pytest.mark.parametrize("trial", range(12))
+def test_random_projection_shapes(gpu, oracle, trial):
+    """Seeded random shapes across both kernels: K any multiple of 256 up to 9216, row counts
+    that are not multiples of a wave's or a workgroup's rows, 1 to 140 tokens."""
+    rng = np.random.default_rng(9100 + trial)
+    K = 256 * int(rng.integers(1, 37))
+    head_dim = int(rng.choice([8, 24, 40, 64, 88, 128]))
+    kv_heads = int(rng.integers(1, 4))
+    heads = kv_heads * int(rng.integers(1, 4))
+    batch = int(rng.choice([1, 2, int(rng.integers(3, 33)), int(rng.integers(33, 65)), int(rng.integers(65, 141))]))
+    say(f"q4k random trial={trial} K={K} heads={heads} kv_heads={kv_heads} head_dim={head_dim} batch={batch}")
+    case = W.make_qkv_projection(seed=9200 + trial, K=K, num_heads=heads, num_kv_heads=kv_heads,
+                                 head_dim=head_dim, batch=batch)
+    yq = dev(np.full((batch, case.Nq), np.nan, np.float32))
+    yk = dev(np.full((batch, case.Nkv), np.nan, np.float32))
+    yv = dev(np.full((batch, case.Nkv), np.nan, np.float32))
+    gpu.fused_qkv_matvec_q4k(dev(case.x), dev(case.wq), dev(case.wk), dev(case.wv), yq, yk, yv, case.K, case.Nq,
+                             case.Nkv, batch=batch)
+    gpu.sync()
+    _check(oracle, yq.read(np.float32, (batch, case.Nq)), case.x, case.wq, "yq")
+    _check(oracle, yk.read(np.float32, (batch, case.Nkv)), case.x, case.wk, "yk")
+    _check(oracle, yv.read(np.float32, (batch, case.Nkv)), case.x, case.wv, "yv")
+
+
 def test_matvec_q4k_output_projection(gpu, oracle):
     """y = Wo x with K = num_heads * head_dim: MetalCompute::matvec_q4k behind attention."""
     rng = np.random.default_rng(3)
