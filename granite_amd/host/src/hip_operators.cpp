@@ -11,8 +11,11 @@
 // columns, which are sliced off again), so the reference's small test tensors
 // (head size 4, tests/test_vulkan.cpp:353-482) go through unchanged.  Shapes:
 //   Q, out  [seq_q, D] | [H, seq_q, D] | [B, H, seq_q, D]   FP16 or FP32
-//   K, V    [seq_kv, D] | [Hkv, seq_kv, D] | [B, Hkv, seq_kv, D]   FP16
-// with H a multiple of Hkv (grouped-query attention).  The extra attribute
+//   K, V    [seq_kv, D] | [Hkv, seq_kv, D] | [B, Hkv, seq_kv, D]   FP16 or FP32
+// with H a multiple of Hkv (grouped-query attention).  The kernels read K and V as halves (the
+// KV cache type); float K and V -- what the reference's operator tests allocate
+// (tests/test_vulkan.cpp:372-374) -- are first rounded to nearest into half temporaries, as the
+// reference's GPU kernels round what they store (metal_shaders_attention.h:124).  The extra attribute
 // `causal` (bool, default true) switches the mask off, which is what the
 // Vulkan operator computes (src/operators/vulkan/vulkan_operators.cpp:392-397).
 #include <cmath>
@@ -64,8 +67,8 @@ class HipAttentionOp final : public IOperator {
             return Error(ErrorCode::ShapeMismatch, "Query heads must be a multiple of KV heads");
         if (Q.dtype() != DataType::FP16 && Q.dtype() != DataType::FP32)
             return Error(ErrorCode::DTypeMismatch, "Q must be FP16 or FP32");
-        if (K.dtype() != DataType::FP16 || V.dtype() != DataType::FP16)
-            return Error(ErrorCode::DTypeMismatch, "K and V must be FP16 (the KV cache type)");
+        if ((K.dtype() != DataType::FP16 && K.dtype() != DataType::FP32) || V.dtype() != K.dtype())
+            return Error(ErrorCode::DTypeMismatch, "K and V must both be FP16 (the KV cache type) or both FP32");
         if (!Q.is_contiguous() || !K.is_contiguous() || !V.is_contiguous())
             return Error(ErrorCode::InvalidArgument, "Q, K and V must be contiguous");
         if (q.dim < 1 || q.dim > 128)
@@ -116,11 +119,40 @@ class HipAttentionOp final : public IOperator {
         const int64_t dim = q.dim == 64 || q.dim == 128 ? q.dim : (q.dim < 64 ? 64 : 128);
         const bool padded = dim != q.dim;
         const uint64_t q_rows = uint64_t(q.batch * q.heads * q.seq), kv_rows = uint64_t(k.batch * k.heads * k.seq);
-        BufferHandle tmp[4] = {};  // Q, K, V, out
+        BufferHandle tmp[6] = {};  // Q, K, V, out (padded); K, V as halves
         auto release = [&] {
             for (BufferHandle& h : tmp)
                 if (h.valid()) ctx.backend->destroy_buffer(h);
         };
+        if (K.dtype() == DataType::FP32) {
+            // [B, Hkv, seq_kv, D] float -> the same layout in halves: per batch entry an append
+            // into a "cache" of exactly seq_kv rows per head, starting at row 0
+            Result<void> status;
+            for (int i = 4; i < 6 && status.ok(); ++i) {
+                auto made = ctx.backend->create_buffer(BufferDesc::device(kv_rows * q.dim * sizeof(uint16_t)));
+                if (!made.ok()) status = made.error();
+                else tmp[i] = made.value();
+            }
+            char* kh = status.ok() ? static_cast<char*>(hip_device_pointer(ctx.backend, tmp[4])) : nullptr;
+            char* vh = status.ok() ? static_cast<char*>(hip_device_pointer(ctx.backend, tmp[5])) : nullptr;
+            const size_t batch_elems = size_t(k.heads * k.seq * q.dim);
+            for (int64_t b = 0; b < k.batch && status.ok(); ++b)
+                status = hip_status_to_result(
+                    granite_hip_kv_cache_append_ex(kh + b * batch_elems * sizeof(uint16_t),
+                                                   vh + b * batch_elems * sizeof(uint16_t),
+                                                   k_ptr + b * batch_elems * sizeof(float),
+                                                   v_ptr + b * batch_elems * sizeof(float), GRANITE_HIP_F32, q.dim,
+                                                   k.seq * q.dim, uint32_t(k.heads), uint32_t(q.dim), 0,
+                                                   uint32_t(k.seq), uint32_t(k.seq), GRANITE_HIP_ROUND_NEAREST),
+                    "granite_hip_kv_cache_append_ex");
+            if (!status.ok()) {
+                release();
+                return status;
+            }
+            k_ptr = kh;
+            v_ptr = vh;
+        }
+        const bool temporaries = padded || K.dtype() == DataType::FP32;
         if (padded) {
             const size_t bytes[4] = {q_rows * dim * q_esz, kv_rows * dim * 2, kv_rows * dim * 2, q_rows * dim * q_esz};
             char* const src[3] = {q_ptr, k_ptr, v_ptr};
@@ -177,11 +209,13 @@ class HipAttentionOp final : public IOperator {
                 return launched;
             }
         }
-        if (padded) {
-            auto sliced = hip_status_to_result(
-                granite_hip_copy_rows(o_ptr, int64_t(q.dim * q_esz), result_ptr, int64_t(dim * q_esz), q_rows,
-                                      uint32_t(q.dim * q_esz), uint32_t(q.dim * q_esz)),
-                "granite_hip_copy_rows");
+        if (temporaries) {
+            Result<void> sliced;
+            if (padded)
+                sliced = hip_status_to_result(
+                    granite_hip_copy_rows(o_ptr, int64_t(q.dim * q_esz), result_ptr, int64_t(dim * q_esz), q_rows,
+                                          uint32_t(q.dim * q_esz), uint32_t(q.dim * q_esz)),
+                    "granite_hip_copy_rows");
             (void)ctx.backend->wait_for_completion();  // the temporaries are released below
             release();
             return sliced;

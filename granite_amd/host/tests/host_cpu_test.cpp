@@ -216,7 +216,10 @@ TEST_CASE(attention_op_validation) {
 
     auto k32 = Tensor::allocate({2, 9, 128}, DataType::FP32, &be).take();
     ctx.inputs = {q, k32, v};
-    CHECK_CODE(op->validate(ctx), ErrorCode::DTypeMismatch);
+    CHECK_CODE(op->validate(ctx), ErrorCode::DTypeMismatch);  // K and V of different types
+    auto v32 = Tensor::allocate({2, 9, 128}, DataType::FP32, &be).take();
+    ctx.inputs = {q, k32, v32};
+    CHECK_OK(op->validate(ctx));  // both float: rounded to half on the way in
     auto k3 = Tensor::allocate({3, 9, 128}, DataType::FP16, &be).take();
     auto v3 = Tensor::allocate({3, 9, 128}, DataType::FP16, &be).take();
     ctx.inputs = {q, k3, v3};

@@ -202,12 +202,18 @@ TEST_CASE(operator_known_answer) {
     auto op = OperatorRegistry::instance().create(OpType::ScaledDotProductAttention,
                                                   BackendType::HIP);
     REQUIRE(op != nullptr);
-    for (DataType qdt : {DataType::FP32, DataType::FP16}) {
+    // all float (the dtypes of tests/test_vulkan.cpp:372-374), float queries over a half cache, all half
+    const DataType cases[3][2] = {{DataType::FP32, DataType::FP32}, {DataType::FP32, DataType::FP16},
+                                  {DataType::FP16, DataType::FP16}};
+    for (const auto& dt : cases) {
+        const DataType qdt = dt[0], kvdt = dt[1];
         OpContext ctx;
         ctx.backend = backend();
         Tensor Q = qdt == DataType::FP32 ? upload({2, 4}, qdt, q) : upload({2, 4}, qdt, to_half(q));
-        ctx.inputs = {Q, upload({3, 4}, DataType::FP16, to_half(k)),
-                      upload({3, 4}, DataType::FP16, to_half(v))};
+        if (kvdt == DataType::FP32)
+            ctx.inputs = {Q, upload({3, 4}, kvdt, k), upload({3, 4}, kvdt, v)};
+        else
+            ctx.inputs = {Q, upload({3, 4}, kvdt, to_half(k)), upload({3, 4}, kvdt, to_half(v))};
         auto shapes = op->infer_shapes(ctx);
         REQUIRE(shapes.ok());
         CHECK((shapes.value()[0] == std::vector<int64_t>{2, 4}));
@@ -262,6 +268,43 @@ TEST_CASE(operator_other_head_sizes_vs_oracle) {
             for (int s = 0; s < seq_q; ++s)
                 std::memcpy(&want[(size_t(h) * seq_q + s) * dim], &want_tok[(size_t(s) * H + h) * dim], dim * 4);
         CHECK(close_enough(got, want, "operator, head size without a kernel"));
+        for (auto& t : ctx.inputs) backend()->destroy_buffer(t.buffer());
+        backend()->destroy_buffer(ctx.outputs[0].buffer());
+    }
+    // float K and V (what the reference's operator tests allocate): a head size with a kernel and
+    // one without, several batch entries; the values are halves widened to float, so that the
+    // oracle's half cache holds exactly what the operator's conversion produces
+    for (int dim : {128, 40}) {
+        const int B = 2, H = 4, Hkv = 2, seq_q = 21, seq_kv = 37, start = seq_kv - seq_q;
+        auto q = randn(size_t(B) * H * seq_q * dim, 700 + dim);                     // [B, H, seq_q, dim]
+        auto kh = to_half(randn(size_t(B) * Hkv * seq_kv * dim, 701 + dim));        // [B, Hkv, seq_kv, dim]
+        auto vh = to_half(randn(size_t(B) * Hkv * seq_kv * dim, 702 + dim));
+        OpContext ctx;
+        ctx.backend = backend();
+        ctx.inputs = {upload({B, H, seq_q, dim}, DataType::FP32, q),
+                      upload({B, Hkv, seq_kv, dim}, DataType::FP32, to_float(kh)),
+                      upload({B, Hkv, seq_kv, dim}, DataType::FP32, to_float(vh))};
+        auto out = Tensor::allocate({B, H, seq_q, dim}, DataType::FP32, backend());
+        REQUIRE(out.ok());
+        ctx.outputs = {out.take()};
+        ctx.attrs.set("start_pos", int64_t(start));
+        CHECK_OK(op->execute(ctx));
+        auto got = download<float>(ctx.outputs[0]);
+        std::vector<float> want(q.size());
+        for (int b = 0; b < B; ++b) {
+            const size_t qo = size_t(b) * H * seq_q * dim, ko = size_t(b) * Hkv * seq_kv * dim;
+            std::vector<float> q_tok(size_t(H) * seq_q * dim), want_tok(q_tok.size());
+            for (int h = 0; h < H; ++h)
+                for (int s = 0; s < seq_q; ++s)
+                    std::memcpy(&q_tok[(size_t(s) * H + h) * dim], &q[qo + (size_t(h) * seq_q + s) * dim], dim * 4);
+            go_attention_cached(q_tok.data(), kh.data() + ko, vh.data() + ko, want_tok.data(), nullptr, 1, seq_q, H,
+                                Hkv, dim, seq_kv, seq_kv, start, 1.0f / std::sqrt(float(dim)));
+            for (int h = 0; h < H; ++h)
+                for (int s = 0; s < seq_q; ++s)
+                    std::memcpy(&want[qo + (size_t(h) * seq_q + s) * dim], &want_tok[(size_t(s) * H + h) * dim],
+                                dim * 4);
+        }
+        CHECK(close_enough(got, want, "operator, float K and V"));
         for (auto& t : ctx.inputs) backend()->destroy_buffer(t.buffer());
         backend()->destroy_buffer(ctx.outputs[0].buffer());
     }
