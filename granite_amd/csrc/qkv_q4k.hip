@@ -322,13 +322,18 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
     // ---- all loads first, the inputs ahead of the weights: loads return in the order they were
     // issued, so the inputs (from the last-level cache) can be converted while the weights are
     // still on their way from HBM
-    float4v raw[kTiles][8];  // thread (token, sub-block) of each tile: 32 inputs
+    // 16 threads per token; thread j of them takes the 16-byte pieces j, j + 16, ... of the
+    // token's 512 columns, so that a load instruction covers 256 contiguous bytes per token
+    // (with the pieces of a sub-block in one thread it touched 16 lines per token for 16 bytes
+    // each, and the vector cache took four times as long over the same bytes)
+    float4v raw[kTiles][8];
 #pragma unroll
     for (int t = 0; t < kTiles; t++) {
         const uint32_t b = t * kTokTile + tid / kSubPerChunk, j = tid % kSubPerChunk;
-        const float* xp = p.x + int64_t(tok0 + min(b, tile_batch - 1)) * p.x_stride + min(k0 + 32 * j, K - 32);
+        const float* xb = p.x + int64_t(tok0 + min(b, tile_batch - 1)) * p.x_stride;
 #pragma unroll
-        for (int i = 0; i < 8; i++) raw[t][i] = *reinterpret_cast<const float4v*>(xp + 4 * i);
+        for (int i = 0; i < 8; i++)
+            raw[t][i] = *reinterpret_cast<const float4v*>(xb + min(k0 + 4 * (j + 16 * i), K - 4));
     }
     uint4v head[kChunkBlocks], nib[kChunkBlocks][4];
     bool live_block[kChunkBlocks];
@@ -343,24 +348,24 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
             nib[sb][G] = __builtin_nontemporal_load(reinterpret_cast<const uint4v*>(blk + 16 + 32 * G + 16 * g));
     }
 
-    // ---- stage the chunk's inputs: thread (token, sub-block) converts 32 floats.  A token's
-    // inputs of this chunk are first scaled by a power of two (exact) that brings the largest
-    // of them into [1, 2), so that the split into a half and a half remainder keeps 22
-    // significant bits of the largest inputs whatever their magnitude -- inputs beyond the
-    // half range and inputs far below its normal range alike -- and a sub-block's sum of 32
-    // inputs stays below 64.  The factor is taken out again when the chunk's products are
-    // added to y.
+    // ---- stage the chunk's inputs.  A token's inputs of this chunk are first scaled by a power
+    // of two (exact) that brings the largest of them into [1, 2), so that the split into a half
+    // and a half remainder keeps 22 significant bits of the largest inputs whatever their
+    // magnitude -- inputs beyond the half range and inputs far below its normal range alike --
+    // and a sub-block's sum of 32 inputs stays below 64.  The factor is taken out again when
+    // the chunk's products are added to y.
+    static_assert(kSubPerChunk == 16 && kChunkK == 512, "16 threads per token, eight 16-byte pieces each");
 #pragma unroll
     for (int t = 0; t < kTiles; t++) {
         const uint32_t b = t * kTokTile + tid / kSubPerChunk, j = tid % kSubPerChunk;
-        const bool live = b < tile_batch && k0 + 32 * j < K;
+        const bool live_token = b < tile_batch;
         float amax = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const float4v v = raw[t][i];
-            if (live) amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+            if (live_token && k0 + 4 * (j + 16 * i) < K)
+                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
         }
-        static_assert(kSubPerChunk == 16, "a token's sub-blocks are 16 neighbouring lanes");
 #pragma unroll
         for (int m = 1; m < kSubPerChunk; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
         // 2^floor(log2 amax), kept inside [2^-126, 2^126] so that it and its inverse are normal floats
@@ -368,14 +373,16 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
         const float unit = amax > 0.0f ? __uint_as_float(ebits) : 1.0f;
         const float scale = 1.0f / unit;
         if (j == 0) s_unit[b] = unit;
-        float sum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float4v a = raw[t][2 * i], c = raw[t][2 * i + 1];
-            const float v[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
-            uint32_t hi[4], lo[4];
+        for (int i = 0; i < 8; i++) {
+            const uint32_t col = 4 * (j + 16 * i);  // first of the piece's four columns
+            const bool live = live_token && k0 + col < K;
+            const float4v r = raw[t][i];
+            const float v[4] = {r.x, r.y, r.z, r.w};
+            uint32_t hi[2], lo[2];
+            float sum = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
+            for (int e = 0; e < 2; e++) {
                 const float x0 = live ? v[2 * e] * scale : 0.0f, x1 = live ? v[2 * e + 1] * scale : 0.0f;
                 sum += x0 + x1;
                 const _Float16 h0 = static_cast<_Float16>(x0), h1 = static_cast<_Float16>(x1);
@@ -387,12 +394,18 @@ __global__ void __launch_bounds__(kTokWaves* kWave, 1) matmul_q4k_tokens_kernel(
                 hi[e] = __builtin_bit_cast(uint32_t, hh);
                 lo[e] = __builtin_bit_cast(uint32_t, ll);
             }
-            *reinterpret_cast<uint4v*>(s_xh + b * kXPitch + 32 * j + 8 * i) = uint4v{hi[0], hi[1], hi[2], hi[3]};
-            *reinterpret_cast<uint4v*>(s_xl + b * kXPitch + 32 * j + 8 * i) = uint4v{lo[0], lo[1], lo[2], lo[3]};
+            *reinterpret_cast<uint2v*>(s_xh + b * kXPitch + col) = uint2v{hi[0], hi[1]};
+            *reinterpret_cast<uint2v*>(s_xl + b * kXPitch + col) = uint2v{lo[0], lo[1]};
+            // the eight pieces of sub-block 2 i + j / 8 lie in eight neighbouring threads
+#pragma unroll
+            for (int m = 1; m < 8; m <<= 1) sum += __shfl_xor(sum, m, kWave);
+            if ((j & 7) == 0) {
+                const _Float16 sh = static_cast<_Float16>(sum);
+                s_sh[b * kSubPerChunk + 2 * i + (j >> 3)] = __builtin_bit_cast(uint16_t, sh);
+                s_sl[b * kSubPerChunk + 2 * i + (j >> 3)] =
+                    __builtin_bit_cast(uint16_t, static_cast<_Float16>(sum - static_cast<float>(sh)));
+            }
         }
-        const _Float16 sh = static_cast<_Float16>(sum);
-        s_sh[b * kSubPerChunk + j] = __builtin_bit_cast(uint16_t, sh);
-        s_sl[b * kSubPerChunk + j] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(sum - static_cast<float>(sh)));
     }
     __syncthreads();
 
