@@ -1,10 +1,11 @@
 // Causal GQA flash-attention prefill, chunked prefill over a paged cache and
 // tree-masked attention for gfx950 (MFMA, K/V tiles staged in LDS): the launcher of
 // granite_hip_attention, the register-staged tiles kernel, the split-K merge and the tree
-// mask kernel.  Launches of head size 128 with no extra key segment and a
-// contiguous cache or blocks of a power of two of at least 8 tokens go to the direct-to-LDS
-// form of the tiles kernel instead (prefill_dma.hip), which shares the grid, the partial
-// layout and the merge; everything else runs the kernel of this file.
+// mask kernel.  Launches of head size 128 with a contiguous cache or blocks of a power of two
+// of at least 8 tokens, and with no extra key segment other than a tree of at most
+// kMaxFusedNodes nodes behind a non-empty cache, go to the direct-to-LDS form of the tiles
+// kernel instead (prefill_dma.hip), which shares the grid, the partial layout and the merge;
+// everything else runs the kernel of this file.
 //
 // Stands in for
 //   flash_attention_prefill     src/backend/metal/kernels/metal_shaders_attention.h:1447-1660
@@ -1002,10 +1003,13 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     const int rows = !a.block_table ? kRowsContiguous
                                     : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
-    // The direct-to-LDS kernel (prefill_dma.hip) where it applies: head size 128, no extra key
-    // segment, contiguous rows or blocks of a power of two >= 8 tokens.
-    bool dma = D == 128 && a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE &&
-                rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3);
+    // The direct-to-LDS kernel (prefill_dma.hip) where it applies: head size 128, contiguous rows
+    // or blocks of a power of two >= 8 tokens, and no extra key segment other than the tree of a
+    // tree-masked launch whose ancestor masks a workgroup builds itself, behind a non-empty cache.
+    const bool tree_dma = a.mask_mode == GRANITE_HIP_MASK_TREE && p.tree_parents != nullptr && a.cache_len > 0 &&
+                          a.extra_len <= kMaxFusedNodes;
+    bool dma = D == 128 && rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3) &&
+               (tree_dma || (a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE));
     if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) dma = dma && e[0] != 't';  // "tiles": the register-staged kernel
     int rc;
     {

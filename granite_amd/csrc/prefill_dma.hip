@@ -44,8 +44,8 @@
 //   (kHandOver; see the loops).
 //
 // Limits (the caller checks them and uses attention_tiles_kernel otherwise): head size 128,
-// no extra key segment (no tree mask), contiguous cache or paged cache with a power-of-two
-// block size >= 8.  Queries fp16 or fp32 (fp32 as an fp16 head and an fp16 remainder: two MFMAs
+// an extra key segment only as the tree of a tree-masked launch of at most kMaxFusedNodes nodes
+// behind a non-empty cache, contiguous cache or paged cache with a power-of-two block size >= 8.  Queries fp16 or fp32 (fp32 as an fp16 head and an fp16 remainder: two MFMAs
 // per step of the scores on one K operand).
 //
 // kRB, the number of 32-row blocks a wave owns, is 1.  With 2 (-DGHIP_DMA_RB=2: four waves of
@@ -115,7 +115,7 @@ __device__ __forceinline__ void wait_transfers() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCount));
 }
 
-template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver>
+template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver, bool kTree>
 __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
     const uint32_t lds0 = uint32_t(uintptr_t((lds_byte*)s_raw));  // LDS address of the tile buffers
@@ -161,7 +161,14 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         const uint32_t q_last = min((late_half + 1) * kHalf, p.seq_q) - 1;
         len_a = min(len_a, p.start_pos + q_last + 1);
     }
-    const uint32_t all_tiles = (len_a + kWBN - 1) / kWBN;
+    // A tree launch (kTree): the tree's own keys, the extra segment [num_kv_heads, extra_len, D],
+    // follow the cache's on the key axis from the next tile boundary on, so that a tile holds
+    // keys of one segment only.  Keys len_a .. pad_a - 1 do not exist (masked like a ragged end);
+    // key pad_a + j is tree node j, visible to a row iff the row's ancestor mask has bit j.
+    const uint32_t len_b = kTree ? p.extra_len : 0u;
+    const uint32_t pad_a = (len_a + kWBN - 1) / kWBN * kWBN;
+    const uint32_t len_v = kTree ? pad_a + len_b : len_a;  // end of the key axis
+    const uint32_t all_tiles = (len_v + kWBN - 1) / kWBN;
     const uint32_t t_begin = uint32_t(uint64_t(all_tiles) * split / p.n_splits);
     const uint32_t n_tiles = uint32_t(uint64_t(all_tiles) * (split + 1) / p.n_splits);
 
@@ -172,7 +179,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     {
         uint32_t vis_end = 0;
         if (wave_active) {
-            vis_end = len_a;
+            vis_end = len_v;
             if (causal) vis_end = min(vis_end, p.start_pos + min(q0 + kWaveRows, p.seq_q));
             vis_end = min(vis_end, n_tiles * kWBN);
         }
@@ -229,10 +236,47 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             for (int r = 0; r < 16; r++) oacc[rb][t][r] = 0.0f;
     }
 
+    // ---- tree launches: the ancestor masks.  Row i has bit j set iff tree node i may attend node
+    // j: itself and its ancestors (src/llm/transformer.mm:822-840).  A workgroup whose share of
+    // the keys reaches the tree's own builds them in LDS from the parent pointers, one thread per
+    // node, at most num_nodes steps, so a malformed array cannot hang it.  The pointers are
+    // requested here and the masks are built in the prologue, behind the first tiles' transfers.
+    __shared__ int32_t s_parent[kTree ? kMaxFusedNodes : 1];
+    __shared__ uint32_t s_rowmask[kTree ? kMaxFusedNodes * (kMaxFusedNodes / 32) : 1];
+    static_assert(!kTree || kMaxFusedNodes <= uint32_t(kWThreads), "one thread per node");
+    const bool build_masks = kTree && t_begin < n_tiles && n_tiles * kWBN > pad_a;  // uniform over the workgroup
+    int32_t my_parent = -1;
+    if constexpr (kTree) {
+        if (build_masks && tid < len_b) my_parent = p.tree_parents[tid];
+    }
+    auto build_tree_masks = [&]() __attribute__((always_inline)) {  // by every thread; leaves one barrier to the caller
+        if (tid < len_b) s_parent[tid] = my_parent;
+        for (uint32_t i = tid; i < len_b * p.mask_words; i += kWThreads) s_rowmask[i] = 0;
+        __syncthreads();
+        if (tid < len_b) {
+            uint32_t* row = s_rowmask + tid * p.mask_words;
+            row[tid >> 5] |= 1u << (tid & 31);
+            int32_t cur = my_parent;
+            for (uint32_t step = 0; step < len_b && cur >= 0 && cur < int32_t(len_b); step++) {
+                row[uint32_t(cur) >> 5] |= 1u << (uint32_t(cur) & 31);
+                cur = s_parent[cur];
+            }
+        }
+    };
+
     // ---- staging.  Wave w moves keys kWaveKeys w .. + kWaveKeys - 1 of a tile.
     const int64_t stride_bytes = p.a_tok_stride * 2;  // between consecutive tokens of one KV head
     const unsigned char* const k_bytes = reinterpret_cast<const unsigned char*>(p.k + size_t(kvh) * p.a_head_stride);
     const unsigned char* const v_bytes = reinterpret_cast<const unsigned char*>(p.v + size_t(kvh) * p.a_head_stride);
+    // the tree's keys of this KV head: rows of 2 D bytes one after the other (null without a tree)
+    const unsigned char* const kx_bytes =
+        kTree ? reinterpret_cast<const unsigned char*>(p.k_extra + size_t(kvh) * len_b * kD) : nullptr;
+    const unsigned char* const vx_bytes =
+        kTree ? reinterpret_cast<const unsigned char*>(p.v_extra + size_t(kvh) * len_b * kD) : nullptr;
+    // byte offset of tree key `key` of the key axis inside them, clamped to the last node
+    auto extra_row = [&](uint32_t key) __attribute__((always_inline)) -> uint64_t {
+        return uint64_t(min(key - pad_a, len_b - 1)) * uint64_t(2 * kD);
+    };
     // K transfer (a, h): key 8 a + (lane >> 3) of the wave's, whose slot lane & 7 receives the 16-byte
     // piece slot ^ key of half h of the row: eight consecutive lanes fetch one 128-byte line
     const uint32_t k_lane_off = uint32_t((lane >> 3) * stride_bytes) + 16 * ((lane & 7) ^ (lane >> 3));
@@ -281,7 +325,15 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     // (unused for a ragged tile)
     auto stage_k = [&](uint32_t sw, uint32_t tile, uint32_t buf, uint32_t row) __attribute__((always_inline)) {
         const uint32_t dst = lds0 + buf * kKTile + (kWaveKeys / 8) * sw * kKChunk;
-        if ((tile + 1) * kWBN <= len_a) {
+        if (kTree && tile * kWBN >= pad_a) {  // a tile of the tree's keys: per-lane addresses
+#pragma unroll
+            for (uint32_t a = 0; a < kWaveKeys / 8; a++) {
+                const unsigned char* src = kx_bytes + extra_row(tile * kWBN + kWaveKeys * sw + 8 * a + (lane >> 3)) +
+                                           16 * ((lane & 7) ^ (lane >> 3));
+                dma_lanes(dst + a * kKChunk, src);
+                dma_lanes(dst + (8 + a) * kKChunk, src + 128);
+            }
+        } else if ((tile + 1) * kWBN <= len_a) {
             const unsigned char* base = k_bytes + uint64_t(__builtin_amdgcn_readfirstlane(row)) * uint64_t(stride_bytes);
 #pragma unroll
             for (uint32_t a = 0; a < kWaveKeys / 8; a++) {
@@ -300,7 +352,12 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     };
     auto stage_v = [&](uint32_t sw, uint32_t tile, uint32_t buf, uint32_t row) __attribute__((always_inline)) {
         const uint32_t dst = lds0 + kVRegion + buf * kVTile + kWaveKeys * sw * 256;
-        if ((tile + 1) * kWBN <= len_a) {
+        if (kTree && tile * kWBN >= pad_a) {
+#pragma unroll
+            for (uint32_t j = 0; j < kWaveKeys / 4; j++)
+                dma_lanes(dst + j * 1024,
+                          vx_bytes + extra_row(tile * kWBN + kWaveKeys * sw + 4 * j + (lane >> 4)) + v_swizzled);
+        } else if ((tile + 1) * kWBN <= len_a) {
             const unsigned char* base = v_bytes + uint64_t(__builtin_amdgcn_readfirstlane(row)) * uint64_t(stride_bytes);
 #pragma unroll
             for (uint32_t j = 0; j < kWaveKeys / 4; j++) dma_rows(dst + j * 1024, base + 4 * j * stride_bytes, v_lane_off);
@@ -358,6 +415,22 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     // keys of sub-tile j that a row may not see become minus infinity
     auto apply_mask = [&](uint32_t j, float16v (&sacc)[kRB]) __attribute__((always_inline)) {
         const uint32_t key0 = 32 * j;
+        if (kTree && key0 >= pad_a) {  // tree keys: inside the tree, and an ancestor of the row (or itself)
+            const uint32_t node0 = key0 - pad_a;  // a multiple of 32
+#pragma unroll
+            for (int rb = 0; rb < kRB; rb++) {
+                const uint32_t w = node0 >> 5;
+                const uint32_t word = w < p.mask_words ? s_rowmask[min(q_row[rb], len_b - 1) * p.mask_words + w] : 0u;
+                const int32_t room = int32_t(len_b) - int32_t(node0 + 4 * g);
+                const uint32_t bits = word >> (4 * g);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int kc = 8 * (r >> 2) + (r & 3);
+                    if (!((room > kc) && ((bits >> kc) & 1u))) sacc[rb][r] = -INFINITY;
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int rb = 0; rb < kRB; rb++) {
             const uint32_t limit = causal ? min(len_a, p.start_pos + q_row[rb] + 1) : len_a;
@@ -539,7 +612,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         const uint32_t first_row = live ? half * kHalf + kWaveRows * (w % kRunWaves) : p.seq_q;
         uint32_t vis_end = 0;
         if (first_row < p.seq_q) {
-            vis_end = len_a;
+            vis_end = len_v;
             if (causal) vis_end = min(vis_end, p.start_pos + min(first_row + kWaveRows, p.seq_q));
             vis_end = min(vis_end, n_tiles * kWBN);
         }
@@ -618,6 +691,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             uint4v* vclear = reinterpret_cast<uint4v*>(s_raw + kVRegion + 3 * kVTile);
 #pragma unroll
             for (uint32_t i = 0; i < kVTile / 16 / kWThreads; i++) vclear[tid + i * kWThreads] = uint4v{0, 0, 0, 0};
+        }
+        if constexpr (kTree) {
+            if (build_masks) build_tree_masks();  // visible after the barrier below
         }
         wait_transfers<0>();
         __syncthreads();
@@ -755,9 +831,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
 }
 
-template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver>
+template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver, bool kTree = false>
 int launch_dma(const AttnParams& p, dim3 grid) {
-    auto kernel = attention_tiles_dma_kernel<kQF32, kOutF32, kPaged, kHandOver>;
+    auto kernel = attention_tiles_dma_kernel<kQF32, kOutF32, kPaged, kHandOver, kTree>;
     static bool configured[kMaxDevices];  // the tile buffers exceed the 64 KiB default limit
     if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(kernel), kDmaLds, configured)) return rc;
     kernel<<<grid, dim3(kWThreads), kDmaLds, ctx().stream>>>(p);
@@ -773,6 +849,9 @@ int launch_dma_shape(const AttnParams& p, dim3 grid) {
     // prefill over 32k tokens: 0.6 % slower with the hand-over compiled in).
     // The same holds when all the rows of a launch fit one run (at most 128 query rows): the other
     // run's waves are idle from the start.
+    // A tree launch (its rows are the tree's nodes, at most kMaxFusedNodes) always takes the
+    // hand-over form: correct for any shape, and its one instantiation per layout is enough.
+    if (p.mask_mode == GRANITE_HIP_MASK_TREE) return launch_dma<kQF32, kOutF32, kPaged, true, true>(p, grid);
     const bool hand_over =
         (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && p.start_pos < p.seq_q) || p.seq_q <= uint32_t(kWBM / 2);
     return hand_over ? launch_dma<kQF32, kOutF32, kPaged, true>(p, grid)
@@ -791,6 +870,14 @@ size_t tiles_dma_lds_bytes() { return kDmaLds; }
 
 int launch_tiles_dma(const AttnParams& p, dim3 grid, bool q_f32, bool out_f32) {
     if (p.table != nullptr && p.bs_shift < 3) return GRANITE_HIP_EUNSUPPORTED;
+    if (p.mask_mode == GRANITE_HIP_MASK_TREE) {
+        // the kernel builds the ancestor masks itself and numbers the tree's keys behind the cache's
+        if (!p.tree_parents || !p.k_extra || !p.v_extra || p.extra_len == 0 || p.extra_len > kMaxFusedNodes ||
+            p.cache_len == 0 || p.seq_q != p.extra_len)
+            return GRANITE_HIP_EUNSUPPORTED;
+    } else if (p.extra_len != 0) {
+        return GRANITE_HIP_EUNSUPPORTED;
+    }
     if (q_f32) return out_f32 ? launch_dma_layout<true, true>(p, grid) : launch_dma_layout<true, false>(p, grid);
     return out_f32 ? launch_dma_layout<false, true>(p, grid) : launch_dma_layout<false, false>(p, grid);
 }

@@ -34,7 +34,7 @@ WORKLOADS = ["paged_decode", "prefill", "chunked_prefill", "tree", "decode_conti
              "qkv_q4k", "copy_calibration"]
 MFMA_BOUND = {"prefill", "chunked_prefill"}
 DOMINANT = {"paged_decode": "decode_stream_kernel", "prefill": "attention_tiles_dma_kernel",
-            "chunked_prefill": "attention_tiles_dma_kernel", "tree": "attention_tiles_kernel",
+            "chunked_prefill": "attention_tiles_dma_kernel", "tree": "attention_tiles_dma_kernel",
             "decode_contiguous": "decode_splitk_kernel", "rope_append": "rope_append_kernel",
             "qkv_q4k": "matvec_q4k_kernel", "copy_calibration": "kv_gather_kernel"}
 

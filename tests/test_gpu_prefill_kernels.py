@@ -175,7 +175,13 @@ def test_short_chunk_default_kernel_and_tiles_kernel(gpu, oracle, prefix, chunk,
 
 @pytest.mark.parametrize("prefix,n,hq,hkv,bs,paged", [(0, 1, 4, 4, 16, True), (0, 40, 8, 2, 16, True),
                                                      (100, 33, 8, 2, 12, True), (2000, 64, 32, 8, 16, True),
-                                                     (700, 64, 8, 2, 16, False), (4096, 20, 4, 1, 1, True)])
+                                                     (700, 64, 8, 2, 16, False), (4096, 20, 4, 1, 1, True),
+                                                     # the direct-to-LDS kernel's tree form: a prefix that ends inside a
+                                                     # tile, on a tile boundary and one key behind it; trees of more
+                                                     # than one tile and of the largest size it builds masks for
+                                                     (63, 64, 8, 2, 16, True), (64, 64, 8, 2, 16, True), (65, 70, 8, 2, 8, True),
+                                                     (3000, 200, 8, 2, 32, True), (1000, 256, 4, 1, 8, True),
+                                                     (130, 129, 8, 2, 16, False), (5, 3, 4, 4, 64, True)])
 def test_tree_default_kernel_and_tiles_kernel(gpu, oracle, prefix, n, hq, hkv, bs, paged):
     """Tree attention (fp32 queries, a prefix in a paged or contiguous cache, the nodes as the
     extra segment), launched as by default and with the register-staged kernel forced."""
@@ -259,3 +265,34 @@ def test_float_queries_both_kernels(gpu, oracle, prefix, chunk, bs, hq, hkv, out
         results[kernel] = (got, got_lse)
     assert np.abs(results["dma"][0] - results["tiles"][0]).max() <= 1e-3
     assert np.abs(results["dma"][1] - results["tiles"][1]).max() <= 1e-5
+
+
+@pytest.mark.parametrize("prefix,n,hq,hkv,bs,paged", [(500, 64, 8, 2, 16, True), (200, 150, 4, 1, 32, False)])
+def test_tree_half_queries_and_output(gpu, oracle, prefix, n, hq, hkv, bs, paged):
+    """Tree attention with half queries and half output (the default kernel's tree form is
+    instantiated for both query and both output types)."""
+    say(f"tree half prefix={prefix} nodes={n} hq={hq} hkv={hkv} bs={bs} paged={paged}")
+    case = W.make_tree(seed=3 * prefix + n, prefix_len=prefix, num_nodes=n, num_heads=hq, num_kv_heads=hkv,
+                       block_size=bs)
+    qh = case.q.astype(np.float16)                                     # [hq, n, 128]
+    q = np.transpose(qh.astype(np.float32), (1, 0, 2))[None]
+    kt = np.transpose(case.k_tree, (1, 0, 2))[None].astype(np.float32)
+    vt = np.transpose(case.v_tree, (1, 0, 2))[None].astype(np.float32)
+    want, want_lse = oracle.attention_tree(q, case.k_pool, case.v_pool, kt, vt, case.parents, prefix, case.scale,
+                                           table=case.block_table, block_size=bs)
+    if paged:
+        cache = dict(k_cache=dev(case.k_pool), v_cache=dev(case.v_pool), block_size=bs,
+                     block_table=dev(case.block_table), max_seq=prefix)
+    else:
+        rows = case.block_table[np.arange(prefix) // bs] * bs + np.arange(prefix) % bs
+        kc = np.ascontiguousarray(np.transpose(case.k_pool[rows], (1, 0, 2)))
+        vc = np.ascontiguousarray(np.transpose(case.v_pool[rows], (1, 0, 2)))
+        cache = dict(k_cache=dev(kc), v_cache=dev(vc), max_seq=prefix)
+    out, lse = dev(np.zeros((hq, n, 128), np.float16)), dev(np.zeros((hq, n), np.float32))
+    gpu.attention(q=dev(qh), q_dtype=F16, q_tok_stride=128, q_head_stride=n * 128, out=out, out_dtype=F16,
+                  out_tok_stride=128, out_head_stride=n * 128, lse=lse, seq_q=n, num_heads=hq, num_kv_heads=hkv,
+                  head_dim=128, scale=case.scale, cache_len=prefix, k_extra=dev(case.k_tree), v_extra=dev(case.v_tree),
+                  extra_len=n, parents=dev(case.parents), mask_mode=MASK_TREE, **cache)
+    gpu.sync()
+    assert_close(out.read(np.float16, (hq, n, 128)).astype(np.float32), np.transpose(want[0], (1, 0, 2)), "out")
+    assert_lse(lse.read(np.float32, (hq, n)), want_lse[0], "lse")
