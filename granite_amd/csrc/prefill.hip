@@ -948,7 +948,43 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
         return GRANITE_HIP_EINVAL;
     }
 
-    const uint32_t q_tiles = (a.seq_q + kBM - 1) / kBM;
+    // Which kernel: the direct-to-LDS one (prefill_dma.hip) where it applies -- head size 128,
+    // contiguous rows or blocks of a power of two >= 8 tokens, and no extra key segment other
+    // than the tree of a tree-masked launch whose ancestor masks a workgroup builds itself,
+    // behind a non-empty cache -- else the register-staged kernel of this file.
+    const int rows = !a.block_table ? kRowsContiguous
+                                    : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
+    const bool tree_dma = a.mask_mode == GRANITE_HIP_MASK_TREE && a.cache_len > 0 && a.extra_len <= kMaxFusedNodes;
+    bool dma = D == 128 && rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3) &&
+               (tree_dma || (a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE));
+    if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) dma = dma && e[0] != 't';  // "tiles": the register-staged kernel
+
+    // A small tree on that kernel: the query heads of a KV group, side by side.  A tree of 64
+    // nodes is two of a workgroup's eight waves; with [heads, nodes, D] dense (one head's rows
+    // right behind the previous head's, in Q, in the output and therefore in the partials and
+    // the log-sum-exp too) `pack` heads of a group are one head of pack x nodes rows to the
+    // kernel, which only has to take a row's node (row mod nodes) for the ancestor mask.  Up to
+    // 128 rows, i.e. one wave per SIMD computing and its idle partner staging for it; the
+    // workgroups that this saves become key splits, so a workgroup's walk is 1 / pack as long.
+    // Behind a long prefix only (8192 tokens and more: 64 nodes over 16 384 tokens 50.7 -> 41.5 us
+    // a step): at 4096 tokens the step takes as long either way and the partials double.
+    constexpr uint32_t kPackFromTiles = 128;
+    uint32_t seq_q = a.seq_q, num_heads = a.num_heads;  // the launch's shape
+    if (dma && tree_dma && (a.cache_len + kBN - 1) / kBN >= kPackFromTiles &&
+        a.q_head_stride == int64_t(a.seq_q) * a.q_tok_stride &&
+        a.out_head_stride == int64_t(a.seq_q) * a.out_tok_stride) {
+        uint32_t pack = 1;
+        while (2 * pack * a.seq_q <= uint32_t(kBM / 2) && p.group % (2 * pack) == 0) pack *= 2;
+        seq_q = pack * a.seq_q;
+        num_heads = a.num_heads / pack;
+        p.seq_q = seq_q;
+        p.num_heads = num_heads;
+        p.group = p.group / pack;
+        p.q_head_stride *= pack;
+        p.out_head_stride *= pack;
+    }
+
+    const uint32_t q_tiles = (seq_q + kBM - 1) / kBM;
     if (q_tiles > 0x7FFFFFFFu / 2 || a.num_heads > 65535u) return GRANITE_HIP_EINVAL;
 
     // Split the keys over several workgroups when (query tiles x heads) alone cannot
@@ -956,7 +992,7 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     uint32_t n_splits = 1;
     {
         const uint32_t cus = ctx().compute_units > 0 ? uint32_t(ctx().compute_units) : 256u;
-        const uint64_t wgs = uint64_t(q_tiles) * a.num_heads;
+        const uint64_t wgs = uint64_t(q_tiles) * num_heads;
         const uint32_t key_tiles = (a.cache_len + kBN - 1) / kBN + (a.extra_len + kBN - 1) / kBN;
         if (wgs < cus) {
             n_splits = uint32_t((cus + wgs - 1) / wgs);
@@ -971,7 +1007,7 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     if (a.mask_mode == GRANITE_HIP_MASK_TREE && !tree) p.tree_parents = a.parents;
     const size_t mask_bytes =
         tree ? (size_t(a.extra_len) * p.mask_words * sizeof(uint32_t) + 255) & ~size_t(255) : 0;
-    const size_t rows_total = n_splits > 1 ? size_t(n_splits) * a.num_heads * a.seq_q : 0;
+    const size_t rows_total = n_splits > 1 ? size_t(n_splits) * num_heads * seq_q : 0;
     const size_t need = mask_bytes + rows_total * (D + 2) * sizeof(float);
     if (scratch.query) {
         *scratch.query = need;
@@ -992,25 +1028,15 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
             p.part_o = reinterpret_cast<float*>(ws + mask_bytes);
             p.part_ml = p.part_o + rows_total * D;
             p.final_out = a.out;
-            p.final_tok_stride = a.out_tok_stride;
-            p.final_head_stride = a.out_head_stride;
+            p.final_tok_stride = p.out_tok_stride;
+            p.final_head_stride = p.out_head_stride;
         }
     }
     p.q_tiles = q_tiles;
     p.n_splits = n_splits;
-    if (uint64_t(q_tiles) * a.num_heads * n_splits > 0x7FFFFFFFull) return GRANITE_HIP_EINVAL;
-    dim3 grid(q_tiles * a.num_heads * n_splits);
-    const int rows = !a.block_table ? kRowsContiguous
-                                    : (p.bs_shift >= 0 ? kRowsPagedPow2 : kRowsPagedAny);
+    if (uint64_t(q_tiles) * num_heads * n_splits > 0x7FFFFFFFull) return GRANITE_HIP_EINVAL;
+    dim3 grid(q_tiles * num_heads * n_splits);
     const bool qf32 = a.q_dtype == GRANITE_HIP_F32, of32 = a.out_dtype == GRANITE_HIP_F32;
-    // The direct-to-LDS kernel (prefill_dma.hip) where it applies: head size 128, contiguous rows
-    // or blocks of a power of two >= 8 tokens, and no extra key segment other than the tree of a
-    // tree-masked launch whose ancestor masks a workgroup builds itself, behind a non-empty cache.
-    const bool tree_dma = a.mask_mode == GRANITE_HIP_MASK_TREE && p.tree_parents != nullptr && a.cache_len > 0 &&
-                          a.extra_len <= kMaxFusedNodes;
-    bool dma = D == 128 && rows != kRowsPagedAny && (rows == kRowsContiguous || p.bs_shift >= 3) &&
-               (tree_dma || (a.extra_len == 0 && a.mask_mode != GRANITE_HIP_MASK_TREE));
-    if (const char* e = std::getenv("GRANITE_HIP_PREFILL_KERNEL")) dma = dma && e[0] != 't';  // "tiles": the register-staged kernel
     int rc;
     {
         KernelTimerScope timer("attention_tiles");
@@ -1022,7 +1048,7 @@ int launch_attention(const granite_hip_attention_args& a, const ScratchSource& s
     {
         KernelTimerScope timer("attention_merge");
         const uint32_t rows_per_group = 256 / (D / 8);
-        dim3 mgrid((a.seq_q + rows_per_group - 1) / rows_per_group, a.num_heads);
+        dim3 mgrid((seq_q + rows_per_group - 1) / rows_per_group, num_heads);
         hipStream_t st = ctx().stream;
         if (D == 128) {
             if (of32) attention_merge_kernel<true, 128><<<mgrid, dim3(256), 0, st>>>(p, n_splits);

@@ -164,7 +164,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     // A tree launch (kTree): the tree's own keys, the extra segment [num_kv_heads, extra_len, D],
     // follow the cache's on the key axis from the next tile boundary on, so that a tile holds
     // keys of one segment only.  Keys len_a .. pad_a - 1 do not exist (masked like a ragged end);
-    // key pad_a + j is tree node j, visible to a row iff the row's ancestor mask has bit j.
+    // key pad_a + j is tree node j, visible to a row iff the row's ancestor mask has bit j.  Query row
+    // r is node r mod extra_len: the launcher lays the rows of several heads of a KV group end to
+    // end when the tree is small (seq_q a multiple of extra_len).
     const uint32_t len_b = kTree ? p.extra_len : 0u;
     const uint32_t pad_a = (len_a + kWBN - 1) / kWBN * kWBN;
     const uint32_t len_v = kTree ? pad_a + len_b : len_a;  // end of the key axis
@@ -420,7 +422,8 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
 #pragma unroll
             for (int rb = 0; rb < kRB; rb++) {
                 const uint32_t w = node0 >> 5;
-                const uint32_t word = w < p.mask_words ? s_rowmask[min(q_row[rb], len_b - 1) * p.mask_words + w] : 0u;
+                // (the launcher may have laid several heads' rows end to end: a row's node is row mod nodes)
+                const uint32_t word = w < p.mask_words ? s_rowmask[(q_row[rb] % len_b) * p.mask_words + w] : 0u;
                 const int32_t room = int32_t(len_b) - int32_t(node0 + 4 * g);
                 const uint32_t bits = word >> (4 * g);
 #pragma unroll
@@ -873,7 +876,7 @@ int launch_tiles_dma(const AttnParams& p, dim3 grid, bool q_f32, bool out_f32) {
     if (p.mask_mode == GRANITE_HIP_MASK_TREE) {
         // the kernel builds the ancestor masks itself and numbers the tree's keys behind the cache's
         if (!p.tree_parents || !p.k_extra || !p.v_extra || p.extra_len == 0 || p.extra_len > kMaxFusedNodes ||
-            p.cache_len == 0 || p.seq_q != p.extra_len)
+            p.cache_len == 0 || p.seq_q % p.extra_len != 0)
             return GRANITE_HIP_EUNSUPPORTED;
     } else if (p.extra_len != 0) {
         return GRANITE_HIP_EUNSUPPORTED;

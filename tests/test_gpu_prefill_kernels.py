@@ -181,7 +181,12 @@ def test_short_chunk_default_kernel_and_tiles_kernel(gpu, oracle, prefix, chunk,
                                                      # than one tile and of the largest size it builds masks for
                                                      (63, 64, 8, 2, 16, True), (64, 64, 8, 2, 16, True), (65, 70, 8, 2, 8, True),
                                                      (3000, 200, 8, 2, 32, True), (1000, 256, 4, 1, 8, True),
-                                                     (130, 129, 8, 2, 16, False), (5, 3, 4, 4, 64, True)])
+                                                     (130, 129, 8, 2, 16, False), (5, 3, 4, 4, 64, True),
+                                                     # small trees behind a long prefix: the heads of a KV group side by
+                                                     # side in one workgroup (two heads of 64 nodes, four of 20, two of
+                                                     # three heads of 40: no packing, 128 rows exactly)
+                                                     (8200, 64, 8, 2, 16, True), (9000, 20, 8, 2, 32, False),
+                                                     (8192, 40, 6, 2, 16, True), (8300, 32, 16, 4, 8, True)])
 def test_tree_default_kernel_and_tiles_kernel(gpu, oracle, prefix, n, hq, hkv, bs, paged):
     """Tree attention (fp32 queries, a prefix in a paged or contiguous cache, the nodes as the
     extra segment), launched as by default and with the register-staged kernel forced."""
