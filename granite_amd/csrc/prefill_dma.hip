@@ -171,8 +171,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     const uint32_t pad_a = (len_a + kWBN - 1) / kWBN * kWBN;
     const uint32_t len_v = kTree ? pad_a + len_b : len_a;  // end of the key axis
     const uint32_t all_tiles = (len_v + kWBN - 1) / kWBN;
-    const uint32_t t_begin = uint32_t(uint64_t(all_tiles) * split / p.n_splits);
-    const uint32_t n_tiles = uint32_t(uint64_t(all_tiles) * (split + 1) / p.n_splits);
+    // (32-bit products: the launcher refuses shapes where tiles x splits does not fit; a 64-bit
+    // division here is a hundred scalar instructions in front of the first load)
+    const uint32_t t_begin = all_tiles * split / p.n_splits;
+    const uint32_t n_tiles = all_tiles * (split + 1) / p.n_splits;
 
     // ---- sub-tiles (32 keys, numbered from key 0) this wave computes: [j_begin, j_end); from
     // j_mask on a sub-tile holds a key some row of the wave must not see
@@ -873,6 +875,9 @@ size_t tiles_dma_lds_bytes() { return kDmaLds; }
 
 int launch_tiles_dma(const AttnParams& p, dim3 grid, bool q_f32, bool out_f32) {
     if (p.table != nullptr && p.bs_shift < 3) return GRANITE_HIP_EUNSUPPORTED;
+    // the kernel's share of the key tiles per split is computed in 32 bits
+    if ((uint64_t(p.cache_len) / kWBN + uint64_t(p.extra_len) / kWBN + 2) * p.n_splits >= (1ull << 32))
+        return GRANITE_HIP_EUNSUPPORTED;
     if (p.mask_mode == GRANITE_HIP_MASK_TREE) {
         // the kernel builds the ancestor masks itself and numbers the tree's keys behind the cache's
         if (!p.tree_parents || !p.k_extra || !p.v_extra || p.extra_len == 0 || p.extra_len > kMaxFusedNodes ||
