@@ -115,8 +115,17 @@ __device__ __forceinline__ void wait_transfers() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCount));
 }
 
-template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver, bool kTree>
+//
+// kSplit (launches of at most 64 query rows, always with kHandOver): a row block is two of a
+// workgroup's eight waves' worth of rows at most, so four of the first run's waves would find
+// two idle.  Instead waves 0 and 1 take the even 32-key sub-tiles of every tile for row blocks 0
+// and 1 and waves 2 and 3 the odd ones for the same rows: one phase per tile and wave instead
+// of two (scores of tile it + 1, softmax of tile it, second product of tile it - 1, each of the
+// wave's own sub-tile), four SIMDs computing instead of two, and the two halves of a row
+// block's (m, l, O) combined through LDS at the end.
+template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver, bool kTree, bool kSplit>
 __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel(AttnParams p) {
+    static_assert(!kSplit || (kHandOver && kRB == 1), "the split form is a hand-over form");
     extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
     const uint32_t lds0 = uint32_t(uintptr_t((lds_byte*)s_raw));  // LDS address of the tile buffers
 
@@ -152,7 +161,10 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     const bool run_live = !second_run || early_half < late_half;
     const uint32_t my_half = causal ? (second_run ? early_half : late_half)
                                     : (second_run ? late_half : early_half);
-    const uint32_t q0 = run_live ? my_half * kHalf + kWaveRows * (wave % kRunWaves) : p.seq_q;
+    // (split form: waves 2 and 3 have the rows of waves 0 and 1)
+    const uint32_t row_wave = kSplit ? wave % 2 : wave % kRunWaves;
+    const uint32_t my_sub = kSplit ? (wave % kRunWaves) / 2 : 0u;  // the sub-tile of every tile a split wave takes
+    const uint32_t q0 = run_live ? my_half * kHalf + kWaveRows * row_wave : p.seq_q;
     const bool wave_active = q0 < p.seq_q;
 
     // ---- keys this workgroup visits: those of its later run
@@ -614,7 +626,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
         const bool second = w >= kRunWaves;
         const bool live = !second || early_half < late_half;
         const uint32_t half = causal ? (second ? early_half : late_half) : (second ? late_half : early_half);
-        const uint32_t first_row = live ? half * kHalf + kWaveRows * (w % kRunWaves) : p.seq_q;
+        const uint32_t first_row = live ? half * kHalf + kWaveRows * (kSplit ? w % 2 : w % kRunWaves) : p.seq_q;
         uint32_t vis_end = 0;
         if (first_row < p.seq_q) {
             vis_end = len_v;
@@ -622,7 +634,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             vis_end = min(vis_end, n_tiles * kWBN);
         }
         const uint32_t end = max((vis_end + 31) / 32, j_begin);  // its j_end
-        return j_begin < end ? min(end / 2, n_tiles - 1) + 1 : t_begin;
+        // (split form: the second product lags a whole tile, so a range that ends in the first
+        // half of a tile needs the tile behind it as well)
+        return j_begin < end ? min((end + (kSplit ? 1u : 0u)) / 2, n_tiles - 1) + 1 : t_begin;
     };
     // (kHandOver false: every wave stages its own share throughout, and the loop carries no test
     // for it; the launcher says which -- handing over pays when the runs end far apart)
@@ -711,6 +725,47 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
 #pragma unroll
             for (int r = 0; r < 16; r++) s0[rb][r] = s1[rb][r] = 0.0f;
         }
+        uint32_t it = t_begin;
+        if constexpr (kSplit) {
+            // ---- the split form: this wave's sub-tile (my_sub) of every tile.  In iteration `it`,
+            // one phase: the scores of tile it + 1 (K buffer B + 1), the softmax of tile it, the
+            // second product of tile it - 1 (V buffer B + 3).  Scores and probabilities alternate
+            // between two sets of registers.
+            auto split_run = [&](auto subc) __attribute__((always_inline)) {
+                constexpr int kSub = decltype(subc)::value;
+                if (2 * t_begin + kSub < j_end) {
+                    scores(0, kSub, s0);
+                    if (2 * t_begin + kSub >= j_mask) apply_mask(2 * t_begin + kSub, s0);
+                }
+                auto split_iteration = [&](auto bc, uint32_t itc, const float16v (&s_in)[kRB], float16v (&s_out)[kRB],
+                                           const half8 (&p_prev)[kRB][2], half8 (&p_out)[kRB][2]) __attribute__((always_inline)) {
+                    constexpr int B = decltype(bc)::value;
+                    const uint32_t jc = 2 * itc + kSub, jn = jc + 2;
+                    const bool staging = itc < partner_first_idle;  // else the partner stages this wave's share
+                    fused_phase(IC<(B + 1) & 3>{}, IC<kSub>{}, IC<(B + 3) & 3>{}, IC<kSub>{}, jn >= j_mask, jc < j_end, jn, s_out,
+                                s_in, p_out, p_prev, [&](int slot) __attribute__((always_inline)) {
+                                    if (slot == 9 && staging) stage_next(mine, itc, (B + 3) & 3, (B + 2) & 3, 0);
+                                    if (slot == 11 && staging) stage_next(mine, itc, (B + 3) & 3, (B + 2) & 3, 1);
+                                });
+                    end_of_tile(itc, staging ? 1 : 0);
+                };
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // (see the plain loop below)
+                if (it < first_idle) {
+                    for (;;) {
+                        split_iteration(IC<0>{}, it, s0, s1, p_old, p_new);
+                        if (++it >= first_idle) break;
+                        split_iteration(IC<1>{}, it, s1, s0, p_new, p_old);
+                        if (++it >= first_idle) break;
+                        split_iteration(IC<2>{}, it, s0, s1, p_old, p_new);
+                        if (++it >= first_idle) break;
+                        split_iteration(IC<3>{}, it, s1, s0, p_new, p_old);
+                        if (++it >= first_idle) break;
+                    }
+                }
+            };
+            if (my_sub == 0) split_run(IC<0>{});
+            else split_run(IC<1>{});
+        } else {
         if (j_begin < j_end) {
             scores(0, 0, s0);
             if (j_begin >= j_mask) apply_mask(j_begin, s0);
@@ -733,7 +788,6 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
                         p_old, p_new, [](int) {});
             end_of_tile(it, staging ? 1 : 0);
         };
-        uint32_t it = t_begin;
         // Every load the compiler knows of is complete here (vmcnt(0), as the builtin so that it
         // is visible to the compiler's own wait insertion): otherwise it carries one as pending
         // into the loop and waits for the memory counter, i.e. for the transfers in flight, in
@@ -751,6 +805,7 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
                 if (++it >= first_idle) break;
             }
         }
+        }  // !kSplit
         // ---- tiles this wave only helps to stage (its rows see none of their keys): its own
         // share, taken back if the partner had it, and the partner's while that wave computes
         if (it < n_tiles) {
@@ -774,7 +829,48 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
             }
         }
         // the second product of the last sub-tile, when the range ends with the last tile
-        if (j_end == 2 * n_tiles && j_end > j_begin) accumulate((n_tiles - 1 - t_begin) & 3, 1, p_old);
+        if constexpr (kSplit) {
+            // (the wave's sub-tile of the last tile; its probabilities are in the set the last
+            // iteration wrote: p_new after an odd number of iterations)
+            if (2 * (n_tiles - 1) + my_sub < j_end && j_end > j_begin) {
+                if ((first_idle - t_begin) & 1) accumulate((n_tiles - 1 - t_begin) & 3, my_sub, p_new);
+                else accumulate((n_tiles - 1 - t_begin) & 3, my_sub, p_old);
+            }
+        } else {
+            if (j_end == 2 * n_tiles && j_end > j_begin) accumulate((n_tiles - 1 - t_begin) & 3, 1, p_old);
+        }
+    }
+
+    // ---- split form: the odd sub-tiles' (m, l, O) of a row block join the even ones' through LDS
+    // (the tile buffers: every transfer has landed and, after the barrier, nobody reads them)
+    if constexpr (kSplit) {
+        float* const mbuf = reinterpret_cast<float*>(s_raw);  // [row block][64 O + m + l][lane]
+        constexpr uint32_t kMergeFloats = (16 * kBlocks + 2) * 64;
+        const bool first_run = wave < kRunWaves;
+        __syncthreads();
+        if (first_run && my_sub == 1) {
+            float* dst = mbuf + row_wave * kMergeFloats + lane;
+#pragma unroll
+            for (int t = 0; t < kBlocks; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) dst[(16 * t + r) * 64] = oacc[0][t][r];
+            dst[16 * kBlocks * 64] = m_ref[0];
+            dst[(16 * kBlocks + 1) * 64] = l_run[0];
+        }
+        __syncthreads();
+        if (first_run && my_sub == 0) {
+            const float* src = mbuf + row_wave * kMergeFloats + lane;
+            const float m2 = src[16 * kBlocks * 64], l2 = src[(16 * kBlocks + 1) * 64];
+            const float m = fmaxf(m_ref[0], m2);
+            const float f1 = fast_exp2(m_ref[0] - m), f2 = fast_exp2(m2 - m);
+#pragma unroll
+            for (int t = 0; t < kBlocks; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[0][t][r] = oacc[0][t][r] * f1 + src[(16 * t + r) * 64] * f2;
+            l_run[0] = l_run[0] * f1 + l2 * f2;
+            m_ref[0] = m;
+        }
+        if (my_sub != 0) return;  // the even sub-tiles' wave writes the rows
     }
 
     if (!wave_active) return;
@@ -836,9 +932,9 @@ __global__ void __launch_bounds__(kWThreads, 2 / kRB) attention_tiles_dma_kernel
     }
 }
 
-template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver, bool kTree = false>
+template <bool kQF32, bool kOutF32, bool kPaged, bool kHandOver, bool kTree = false, bool kSplit = false>
 int launch_dma(const AttnParams& p, dim3 grid) {
-    auto kernel = attention_tiles_dma_kernel<kQF32, kOutF32, kPaged, kHandOver, kTree>;
+    auto kernel = attention_tiles_dma_kernel<kQF32, kOutF32, kPaged, kHandOver, kTree, kSplit>;
     static bool configured[kMaxDevices];  // the tile buffers exceed the 64 KiB default limit
     if (int rc = raise_dynamic_lds_limit(reinterpret_cast<const void*>(kernel), kDmaLds, configured)) return rc;
     kernel<<<grid, dim3(kWThreads), kDmaLds, ctx().stream>>>(p);
@@ -856,7 +952,12 @@ int launch_dma_shape(const AttnParams& p, dim3 grid) {
     // run's waves are idle from the start.
     // A tree launch (its rows are the tree's nodes, at most kMaxFusedNodes) always takes the
     // hand-over form: correct for any shape, and its one instantiation per layout is enough.
-    if (p.mask_mode == GRANITE_HIP_MASK_TREE) return launch_dma<kQF32, kOutF32, kPaged, true, true>(p, grid);
+    // At most 64 rows: the split form (two waves per row block, each a sub-tile of every tile).
+    const bool split = p.seq_q <= uint32_t(kWBM / 4);
+    if (p.mask_mode == GRANITE_HIP_MASK_TREE)
+        return split ? launch_dma<kQF32, kOutF32, kPaged, true, true, true>(p, grid)
+                     : launch_dma<kQF32, kOutF32, kPaged, true, true, false>(p, grid);
+    if (split) return launch_dma<kQF32, kOutF32, kPaged, true, false, true>(p, grid);
     const bool hand_over =
         (p.mask_mode == GRANITE_HIP_MASK_CAUSAL && p.start_pos < p.seq_q) || p.seq_q <= uint32_t(kWBM / 2);
     return hand_over ? launch_dma<kQF32, kOutF32, kPaged, true>(p, grid)

@@ -78,7 +78,11 @@ def test_paged_chunk_both_kernels(gpu, oracle, prefix, chunk, bs, hq, hkv, out_d
                                                      (513, 8, 8, 520, MASK_CAUSAL), (200, 4, 2, 256, MASK_NONE),
                                                      # no mask and at most 128 rows: the empty run's waves
                                                      # stage for the others from the first tile on
-                                                     (100, 4, 2, 128, MASK_NONE), (128, 8, 8, 300, MASK_NONE)])
+                                                     (100, 4, 2, 128, MASK_NONE), (128, 8, 8, 300, MASK_NONE),
+                                                     # at most 64 rows: two waves per row block, a sub-tile of every
+                                                     # tile each (causal from the start, and unmasked)
+                                                     (33, 4, 2, 40, MASK_CAUSAL), (64, 8, 2, 100, MASK_NONE),
+                                                     (20, 4, 4, 64, MASK_NONE), (47, 2, 1, 47, MASK_NONE)])
 def test_contiguous_both_kernels(gpu, oracle, seq, hq, hkv, max_seq, mask):
     say(f"prefill kernels contiguous seq={seq} hq={hq} hkv={hkv} max_seq={max_seq} mask={mask}")
     case = W.make_prefill(seed=5 * seq + hq, seq=seq, num_heads=hq, num_kv_heads=hkv, max_seq=max_seq)
