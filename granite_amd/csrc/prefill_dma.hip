@@ -43,10 +43,16 @@
 //   partner, alone on its SIMD and bound by its own instruction stream, issues no transfer
 //   (kHandOver; see the loops).
 //
+// * Tree-masked launches (kTree): the tree's own keys follow the cache's on the key axis from the
+//   next tile boundary on and are staged with per-lane addresses; the rows' ancestor masks are
+//   built in LDS from the parent pointers.  Launches of at most 64 rows (kSplit): two waves per
+//   row block, each a sub-tile of every tile.  Both are described at the kernel.
+//
 // Limits (the caller checks them and uses attention_tiles_kernel otherwise): head size 128,
 // an extra key segment only as the tree of a tree-masked launch of at most kMaxFusedNodes nodes
-// behind a non-empty cache, contiguous cache or paged cache with a power-of-two block size >= 8.  Queries fp16 or fp32 (fp32 as an fp16 head and an fp16 remainder: two MFMAs
-// per step of the scores on one K operand).
+// behind a non-empty cache, contiguous cache or paged cache with a power-of-two block size >= 8.
+// Queries fp16 or fp32 (fp32 as an fp16 head and an fp16 remainder: two MFMAs per step of the
+// scores on one K operand).
 //
 // kRB, the number of 32-row blocks a wave owns, is 1.  With 2 (-DGHIP_DMA_RB=2: four waves of
 // 64 rows, one per SIMD) an LDS operand read feeds two MFMAs; that form needs 434 registers per
